@@ -1,0 +1,162 @@
+/*
+ * sdv2kv — C ABI of the MI355X (gfx950) ring-buffer KV-cache path for the
+ * causal Wan DiT of StreamDiffusionV2.
+ *
+ * Two operators, both enqueued on a caller-supplied HIP stream, both working
+ * on caller-owned device memory (the library owns nothing and, apart from the
+ * lazily created constant RoPE state it is handed, keeps no mutable state):
+ *
+ *   sdv2_kv_append_rope  fused RoPE-on-write chunk append
+ *   sdv2_swa_attn_fwd    chunk-Q x (sink + window) K/V flash attention
+ *
+ * Tensors are addressed as [rows, tokens, heads, 128] with explicit element
+ * strides for the first three dimensions; the last dimension is contiguous.
+ * This lets one binary serve the reference's token-major cache
+ * ([B, cap, H, 128], models/wan/causal_stream_inference.py:98-100) and the
+ * head-major physical layout ([B, H, cap, 128] exposed as a permuted view)
+ * that the kernels prefer.
+ *
+ * All functions return SDV2_OK (0) or a negative sdv2_status; they never
+ * throw, never synchronise the device and never allocate device memory.
+ */
+#ifndef SDV2KV_H
+#define SDV2KV_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SDV2KV_ABI_VERSION 1
+#define SDV2_HEAD_DIM 128      /* causal_stream_inference.py:99-100 fixes 128 */
+#define SDV2_MAX_ROWS 16       /* rows (B) per sdv2_kv_append_rope call       */
+
+typedef enum sdv2_status {
+  SDV2_OK = 0,
+  SDV2_ERR_INVALID_ARG = -1,   /* null pointer, bad shape, misaligned stride  */
+  SDV2_ERR_UNSUPPORTED = -2,   /* head_dim != 128, unknown dtype              */
+  SDV2_ERR_OUT_OF_RANGE = -3,  /* write range outside the cache, RoPE row     */
+                               /* beyond the table                            */
+  SDV2_ERR_WORKSPACE = -4,     /* split-KV workspace missing or too small     */
+  SDV2_ERR_LAUNCH = -5         /* hipLaunchKernel reported an error           */
+} sdv2_status;
+
+typedef enum sdv2_dtype {
+  SDV2_BF16 = 0,
+  SDV2_F32 = 1                 /* append only (CPU-plumbing config of the     */
+                               /* reference runs fp32); attention is bf16     */
+} sdv2_dtype;
+
+/* element strides of a [rows, tokens, heads, 128] tensor */
+typedef struct sdv2_stride3 {
+  int64_t row;
+  int64_t token;
+  int64_t head;
+} sdv2_stride3;
+
+int sdv2_abi_version(void);
+const char* sdv2_status_string(int status);
+
+/* ------------------------------------------------------------------------
+ * Fused RoPE-on-write chunk append.
+ *
+ * Replaces, for one transformer layer, the reference's
+ *   causal_rope_apply(q), causal_rope_apply(k)   models/wan/causal_model.py:253-266 (-> :94-108)
+ *   kv_cache["k"|"v"][i, a:b] = ...              models/wan/causal_model.py:321-322, 336-337
+ *   kv_cache["global_end_index"|"local_end_index"][i].fill_(...)   :339-342
+ *
+ * For every row i and chunk token t (grid position (f,h,w) row-major,
+ * absolute frame start_frame[i] + f):
+ *   q_out[i,t]              = rope(q_in[i,t])
+ *   k_cache[i,dst_start[i]+t] = rope(k_in[i,t])
+ *   v_cache[i,dst_start[i]+t] = v_in[i,t]
+ * rope() multiplies the 64 interleaved (even, odd) pairs of each head by the
+ * complex128 table entry in IEEE double without fused multiply-add and rounds
+ * double -> float (-> bfloat16, nearest-even), which is what the reference's
+ * float64 complex multiply followed by .type_as() produces.  Pair p uses
+ * table row `frame` for p < 22, `h` for 22 <= p < 43 and `w` for p >= 43, at
+ * column p (causal_model.py:64-68, 77-78).
+ *
+ * Which slot a chunk lands in (dst_start) and the new index values are
+ * decided by the caller's ring state machine (causal_model.py:302-342); the
+ * kernel only performs the scatter and stores the two int64 indices, so
+ * eviction costs nothing beyond the write of the new chunk.
+ * ---------------------------------------------------------------------- */
+typedef struct sdv2_append_params {
+  const void* q_in;            /* [B,S,H,128]; may be NULL together with q_out */
+  const void* k_in;
+  const void* v_in;
+  void* q_out;                 /* [B,S,H,128] roped query                      */
+  void* k_cache;               /* [B,cap,H,128]                                */
+  void* v_cache;
+  sdv2_stride3 q_in_stride, k_in_stride, v_in_stride;
+  sdv2_stride3 q_out_stride, k_cache_stride, v_cache_stride;
+  const double* freqs;         /* device, complex128 [freq_rows, 64] as (re,im) */
+  int32_t freq_rows;
+  int32_t dtype;               /* sdv2_dtype of all six tensors                */
+  int32_t rows, tokens, heads, head_dim;          /* B, S, H, 128              */
+  int32_t grid_f, grid_h, grid_w;                 /* tokens == f*h*w           */
+  int64_t cache_tokens;                           /* cap                       */
+  const int64_t* start_frame;  /* host [B]: current_start // (h*w)             */
+  const int64_t* dst_start;    /* host [B]: first cache token written          */
+  int64_t* global_end_index;   /* device int64 [B], may be NULL                */
+  int64_t* local_end_index;    /* device int64 [B], may be NULL                */
+  const int64_t* new_global_end;  /* host [B] values stored by the kernel      */
+  const int64_t* new_local_end;   /* host [B]                                  */
+  void* stream;                /* hipStream_t                                  */
+} sdv2_append_params;
+
+int sdv2_kv_append_rope(const sdv2_append_params* p);
+
+/* ------------------------------------------------------------------------
+ * Sliding-window (sink + window) attention of the chunk's queries against
+ * the cache, read in place in physical slot order.
+ *
+ * Replaces flash_attn_interface.flash_attn_with_kvcache(q=, k_cache=,
+ * v_cache=, cache_seqlens=) as called at models/wan/causal_model.py:353-358
+ * and its SDPA fallback attention_with_kvcache_fallback (:111-157):
+ *   out[i] = softmax(q[i] k_cache[i,:seq_lens[i]]^T / sqrt(128)) v_cache[i,:seq_lens[i]]
+ * with no mask inside the chunk (causal=False) and keys at or beyond
+ * seq_lens[i] ignored.  bf16 in, fp32 accumulation, bf16 out.
+ *
+ * Long caches are split over key ranges to fill the 256 CUs; partial results
+ * go through `workspace` (size from sdv2_swa_attn_workspace_bytes) and are
+ * merged by a second kernel on the same stream.
+ * ---------------------------------------------------------------------- */
+typedef struct sdv2_attn_params {
+  const void* q;               /* [B,S,H,128] bf16 (roped)                     */
+  const void* k_cache;         /* [B,L,H,128] bf16 view of the cache           */
+  const void* v_cache;
+  void* out;                   /* [B,S,H,128] bf16                             */
+  const int32_t* seq_lens;     /* device int32 [B]; NULL = every row uses L    */
+  sdv2_stride3 q_stride, k_stride, v_stride, out_stride;
+  int32_t rows, q_tokens, heads, head_dim;        /* B, S, H, 128              */
+  int32_t max_seq_len;                            /* L = k_cache.shape[1]      */
+  int32_t num_splits;          /* 0 = choose from the shape                    */
+  float softmax_scale;         /* <= 0 selects 1/sqrt(head_dim)                */
+  void* workspace;             /* device scratch, 256-byte aligned             */
+  size_t workspace_bytes;
+  void* stream;                /* hipStream_t                                  */
+} sdv2_attn_params;
+
+/* number of key-range splits the library would pick for this shape */
+int sdv2_swa_attn_default_splits(int32_t rows, int32_t q_tokens, int32_t heads, int32_t max_seq_len);
+/* bytes of workspace needed for `num_splits` (0 = default); 0 when unsplit */
+size_t sdv2_swa_attn_workspace_bytes(int32_t rows, int32_t q_tokens, int32_t heads,
+                                     int32_t max_seq_len, int32_t num_splits);
+int sdv2_swa_attn_fwd(const sdv2_attn_params* p);
+
+/* ------------------------------------------------------------------------
+ * Plain device-to-device copy of `bytes` bytes with the library's own 16-byte
+ * vector kernel.  No counterpart in the reference: it exists so that hardware
+ * counters (bytes fetched / written per dispatch) can be scaled against a
+ * kernel whose traffic is known exactly.
+ * ---------------------------------------------------------------------- */
+int sdv2_copy_bytes(void* dst, const void* src, size_t bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SDV2KV_H */

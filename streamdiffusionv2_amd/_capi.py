@@ -1,0 +1,121 @@
+"""ctypes binding of the sdv2kv C ABI (include/sdv2kv.h).
+
+The shared library is the product: there is no Python or CPU fallback.  When
+it is missing, :func:`lib` raises ImportError with the build command.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from pathlib import Path
+from typing import Optional
+
+LIB_PATH = Path(__file__).resolve().parent / "_lib" / "libsdv2kv.so"
+
+ABI_VERSION = 1
+HEAD_DIM = 128
+MAX_ROWS = 16
+
+SDV2_OK = 0
+SDV2_ERR_INVALID_ARG = -1
+SDV2_ERR_UNSUPPORTED = -2
+SDV2_ERR_OUT_OF_RANGE = -3
+SDV2_ERR_WORKSPACE = -4
+SDV2_ERR_LAUNCH = -5
+
+DTYPE_BF16 = 0
+DTYPE_F32 = 1
+
+# every symbol include/sdv2kv.h declares
+EXPORTED_SYMBOLS = (
+    "sdv2_abi_version",
+    "sdv2_status_string",
+    "sdv2_kv_append_rope",
+    "sdv2_swa_attn_default_splits",
+    "sdv2_swa_attn_workspace_bytes",
+    "sdv2_swa_attn_fwd",
+    "sdv2_copy_bytes",
+)
+
+
+class Stride3(C.Structure):
+    _fields_ = [("row", C.c_int64), ("token", C.c_int64), ("head", C.c_int64)]
+
+
+class AppendParams(C.Structure):
+    _fields_ = [
+        ("q_in", C.c_void_p), ("k_in", C.c_void_p), ("v_in", C.c_void_p),
+        ("q_out", C.c_void_p), ("k_cache", C.c_void_p), ("v_cache", C.c_void_p),
+        ("q_in_stride", Stride3), ("k_in_stride", Stride3), ("v_in_stride", Stride3),
+        ("q_out_stride", Stride3), ("k_cache_stride", Stride3), ("v_cache_stride", Stride3),
+        ("freqs", C.c_void_p),
+        ("freq_rows", C.c_int32),
+        ("dtype", C.c_int32),
+        ("rows", C.c_int32), ("tokens", C.c_int32), ("heads", C.c_int32), ("head_dim", C.c_int32),
+        ("grid_f", C.c_int32), ("grid_h", C.c_int32), ("grid_w", C.c_int32),
+        ("cache_tokens", C.c_int64),
+        ("start_frame", C.POINTER(C.c_int64)),
+        ("dst_start", C.POINTER(C.c_int64)),
+        ("global_end_index", C.c_void_p),
+        ("local_end_index", C.c_void_p),
+        ("new_global_end", C.POINTER(C.c_int64)),
+        ("new_local_end", C.POINTER(C.c_int64)),
+        ("stream", C.c_void_p),
+    ]
+
+
+class AttnParams(C.Structure):
+    _fields_ = [
+        ("q", C.c_void_p), ("k_cache", C.c_void_p), ("v_cache", C.c_void_p), ("out", C.c_void_p),
+        ("seq_lens", C.c_void_p),
+        ("q_stride", Stride3), ("k_stride", Stride3), ("v_stride", Stride3), ("out_stride", Stride3),
+        ("rows", C.c_int32), ("q_tokens", C.c_int32), ("heads", C.c_int32), ("head_dim", C.c_int32),
+        ("max_seq_len", C.c_int32),
+        ("num_splits", C.c_int32),
+        ("softmax_scale", C.c_float),
+        ("workspace", C.c_void_p),
+        ("workspace_bytes", C.c_size_t),
+        ("stream", C.c_void_p),
+    ]
+
+
+_LIB: Optional[C.CDLL] = None
+
+
+def lib() -> C.CDLL:
+    """Load libsdv2kv.so once and declare the prototypes."""
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    if not LIB_PATH.exists():
+        raise ImportError(
+            f"{LIB_PATH} is missing: the KV-cache path has no fallback. Build it with "
+            "`python -m streamdiffusionv2_amd.build_ext` (needs ROCm hipcc)."
+        )
+    handle = C.CDLL(str(LIB_PATH))
+    handle.sdv2_abi_version.restype = C.c_int
+    handle.sdv2_abi_version.argtypes = []
+    handle.sdv2_status_string.restype = C.c_char_p
+    handle.sdv2_status_string.argtypes = [C.c_int]
+    handle.sdv2_kv_append_rope.restype = C.c_int
+    handle.sdv2_kv_append_rope.argtypes = [C.POINTER(AppendParams)]
+    handle.sdv2_swa_attn_default_splits.restype = C.c_int
+    handle.sdv2_swa_attn_default_splits.argtypes = [C.c_int32] * 4
+    handle.sdv2_swa_attn_workspace_bytes.restype = C.c_size_t
+    handle.sdv2_swa_attn_workspace_bytes.argtypes = [C.c_int32] * 5
+    handle.sdv2_swa_attn_fwd.restype = C.c_int
+    handle.sdv2_swa_attn_fwd.argtypes = [C.POINTER(AttnParams)]
+    handle.sdv2_copy_bytes.restype = C.c_int
+    handle.sdv2_copy_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+    if handle.sdv2_abi_version() != ABI_VERSION:
+        raise ImportError(
+            f"{LIB_PATH} has ABI version {handle.sdv2_abi_version()}, expected {ABI_VERSION}: rebuild it"
+        )
+    _LIB = handle
+    return handle
+
+
+def check(status: int, what: str) -> None:
+    """Map a C status to the reference's error convention (RuntimeError)."""
+    if status != SDV2_OK:
+        msg = lib().sdv2_status_string(status).decode()
+        raise RuntimeError(f"{what} failed: {msg} (status {status})")

@@ -1,0 +1,162 @@
+"""``CausalWanSelfAttention`` with the KV-cache path on the sdv2kv kernels.
+
+Same constructor, attributes and ``forward`` signature as the reference module
+(models/wan/causal_model.py:160-200), so a block can hold it unchanged:
+``sink_size``, ``adapt_sink_thr`` and ``evict_idx`` are plain attributes set
+and copied from outside (causal_stream_inference.py:95-96,
+demo/vid2vid.py:150-156).  The projections and RMS norms around the path are
+ordinary PyTorch modules; the path itself (RoPE, ring append, attention) is
+two HIP kernels and no device-to-host copy.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+import torch.nn as nn
+
+from . import ops, ring
+
+
+class WanRMSNorm(nn.Module):
+    """RMS norm over the full model dim in fp32 (wan_base/modules/model.py:70-86)."""
+
+    def __init__(self, dim: int, eps: float = 1e-5):
+        super().__init__()
+        self.dim = dim
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(dim))
+
+    def forward(self, x):
+        xf = x.float()
+        return (xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + self.eps)).type_as(x) * self.weight
+
+
+_HOST_LIST_CACHE: dict = {}
+
+
+def _host_ints(value, slot: str, rows: Optional[int] = None) -> List[int]:
+    """``current_start`` / ``grid_sizes`` as python ints.  A device tensor costs
+    one copy per distinct (tensor, version): the same tensor is handed to every
+    layer of a forward, so all but the first layer hit the one-entry cache."""
+    if isinstance(value, torch.Tensor):
+        if value.device.type == "cpu":
+            out = value.reshape(-1).tolist()
+        else:
+            stamp = (value._version, value.data_ptr(), tuple(value.shape))
+            hit = _HOST_LIST_CACHE.get(slot)
+            if hit is not None and hit[0] is value and hit[1] == stamp:
+                out = hit[2]
+            else:
+                out = value.reshape(-1).tolist()
+                _HOST_LIST_CACHE[slot] = (value, stamp, out)
+    elif isinstance(value, (list, tuple)):
+        out = list(value)
+    else:
+        out = [value]
+    out = [int(x) for x in out]
+    if rows is not None and len(out) == 1 and rows > 1:
+        out = out * rows
+    return out
+
+
+class CausalWanSelfAttention(nn.Module):
+
+    def __init__(self, dim, num_heads, window_size=(-1, -1), qk_norm=True, eps=1e-6):
+        assert dim % num_heads == 0
+        super().__init__()
+        self.dim = dim
+        self.num_heads = num_heads
+        self.head_dim = dim // num_heads
+        self.window_size = window_size
+        self.qk_norm = qk_norm
+        self.eps = eps
+
+        # ring state, same defaults as causal_model.py:177-179
+        self.sink_size = 3
+        self.adapt_sink_thr = -1
+        self.evict_idx: Optional[List[List[int]]] = None
+
+        self.q = nn.Linear(dim, dim)
+        self.k = nn.Linear(dim, dim)
+        self.v = nn.Linear(dim, dim)
+        self.o = nn.Linear(dim, dim)
+        self.norm_q = WanRMSNorm(dim, eps=eps) if qk_norm else nn.Identity()
+        self.norm_k = WanRMSNorm(dim, eps=eps) if qk_norm else nn.Identity()
+
+    # ------------------------------------------------------------------
+    def forward(
+        self,
+        x,
+        seq_lens,
+        grid_sizes,
+        freqs,
+        block_mask,
+        kv_cache=None,
+        current_start=0,
+        current_end=0,
+        causal_rope_cache=None,
+    ):
+        """x [B, S, dim]; grid_sizes [B, 3] = (F, H, W); freqs complex128
+        [1024, head_dim/2]; ``current_end`` and ``causal_rope_cache`` are
+        accepted and unused, as ``current_end`` is in the reference (:281)."""
+        if kv_cache is None:
+            raise NotImplementedError(
+                "only the KV-cache inference path is built; the cache-less flex-attention "
+                "training path (causal_model.py:220-249) is out of scope"
+            )
+        b, s, n, d = *x.shape[:2], self.num_heads, self.head_dim
+        q = self.norm_q(self.q(x)).view(b, s, n, d)
+        k = self.norm_k(self.k(x)).view(b, s, n, d)
+        v = self.v(x).view(b, s, n, d)
+        out = self.attend(q, k, v, grid_sizes, freqs, kv_cache, current_start)
+        return self.o(out.flatten(2))
+
+    # ------------------------------------------------------------------
+    def attend(self, q, k, v, grid_sizes, freqs, kv_cache, current_start,
+               return_roped_query: bool = False):
+        """The path proper, after the projections: RoPE + ring append +
+        attention for q/k/v [B, S, H, 128] (causal_model.py:250-384)."""
+        rows = q.shape[0]
+        grids = _host_ints(grid_sizes, "grid")
+        f, h, w = grids[0], grids[1], grids[2]
+        for r in range(1, len(grids) // 3):
+            if tuple(grids[3 * r:3 * r + 3]) != (f, h, w):
+                raise RuntimeError("all rows of a call must share one (F, H, W) grid")
+        frame_tokens = h * w
+        starts = _host_ints(current_start, "start", rows)
+        if len(starts) != rows:
+            raise RuntimeError(f"current_start has {len(starts)} entries for {rows} rows")
+
+        cache_rows = kv_cache["k"].shape[0]
+        if self.evict_idx is None:
+            self.evict_idx = [[]]
+        if len(self.evict_idx) < cache_rows:
+            self.evict_idx = [list(self.evict_idx[0]) for _ in range(cache_rows)]
+
+        if self.sink_size * frame_tokens > 0 and self.adapt_sink_thr > -1 and q.shape[1] <= frame_tokens:
+            raise NotImplementedError(
+                "adaptive sink refresh (causal_model.py:284-299) is not built yet; "
+                "set adapt_sink_thr = -1 for permanent sinks"
+            )
+
+        plan = ring.plan_append(kv_cache, self.evict_idx, starts, q.shape[1], frame_tokens, self.sink_size)
+        table = ops.device_freqs(freqs, q.device)
+        roped_q = ops.kv_append_rope(
+            q, k, v, kv_cache["k"], kv_cache["v"], table, (f, h, w),
+            [c // frame_tokens for c in starts], plan.dst_start,
+            global_end_index=kv_cache["global_end_index"],
+            local_end_index=kv_cache["local_end_index"],
+            new_global_end=plan.new_global_end,
+            new_local_end=plan.new_local_end,
+        )
+        span = plan.max_seq_len
+        seq = None
+        if any(n != span for n in plan.new_local_end):
+            # rows differ only while the stream batch is still filling; the
+            # lengths are a handful of host ints, shipped asynchronously
+            seq = torch.tensor(plan.new_local_end, dtype=torch.int32).to(q.device, non_blocking=True)
+        out = ops.swa_attention(roped_q, kv_cache["k"][:, :span], kv_cache["v"][:, :span], seq)
+        if return_roped_query:
+            return out, roped_q
+        return out

@@ -1,0 +1,243 @@
+// Fused RoPE-on-write chunk append for gfx950.
+//
+// One launch per transformer layer rotates the chunk's Q and K in IEEE double
+// (no fused multiply-add), rounds double -> float (-> bf16 nearest-even),
+// scatters K' and V into the ring slot chosen by the host state machine and
+// stores the two int64 end indices.  It stands in for causal_rope_apply x2
+// plus the per-row slice writes and index fills of
+// models/wan/causal_model.py:253-266, 321-322, 336-342.
+//
+// The kernel is a pure stream: 16-byte loads and stores, 16 lanes per
+// 256-byte head row, several heads per thread so the four table entries a
+// lane needs are fetched once and reused.  Algorithmic traffic per launch is
+// 6*B*S*H*128*sizeof(T) bytes (read q,k,v; write q', k', v).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "sdv2kv.h"
+#include "sdv2kv_internal.h"
+
+namespace {
+
+constexpr int kLanesPerRow = 16;            // 16 lanes x 8 elements = 128
+constexpr int kTokensPerBlock = 16;         // 256 threads
+constexpr int kHeadsPerThread = 4;
+
+struct AppendKernelArgs {
+  const void* q_in;
+  const void* k_in;
+  const void* v_in;
+  void* q_out;
+  void* k_cache;
+  void* v_cache;
+  sdv2_stride3 q_in_st, k_in_st, v_in_st, q_out_st, k_st, v_st;
+  const double2* freqs;
+  int64_t* global_end;
+  int64_t* local_end;
+  int32_t tokens, heads, grid_w, frame_tokens;
+  int32_t split_t, split_h;                 // pair index bounds: [0,split_t) temporal, [split_t,split_h) height
+  int32_t pairs;                            // 64
+  int64_t start_frame[SDV2_MAX_ROWS];
+  int64_t dst_start[SDV2_MAX_ROWS];
+  int64_t new_global[SDV2_MAX_ROWS];
+  int64_t new_local[SDV2_MAX_ROWS];
+};
+
+template <typename T>
+struct Vec8;
+
+template <>
+struct Vec8<uint16_t> {                     // bf16 bit patterns
+  uint4 raw;
+  __device__ static Vec8 load(const uint16_t* p) {
+    Vec8 v;
+    v.raw = *reinterpret_cast<const uint4*>(p);
+    return v;
+  }
+  __device__ void store(uint16_t* p) const { *reinterpret_cast<uint4*>(p) = raw; }
+  __device__ double get(int i) const {
+    const uint32_t w = (&raw.x)[i >> 1];
+    const uint32_t bits = (i & 1) ? (w & 0xffff0000u) : (w << 16);
+    return static_cast<double>(__uint_as_float(bits));
+  }
+  __device__ void set_pair(int p, double re, double im) {
+    (&raw.x)[p] = sdv2::f32_to_bf16_rne(static_cast<float>(re)) |
+                  (sdv2::f32_to_bf16_rne(static_cast<float>(im)) << 16);
+  }
+};
+
+template <>
+struct Vec8<float> {
+  float4 lo, hi;
+  __device__ static Vec8 load(const float* p) {
+    Vec8 v;
+    v.lo = *reinterpret_cast<const float4*>(p);
+    v.hi = *reinterpret_cast<const float4*>(p + 4);
+    return v;
+  }
+  __device__ void store(float* p) const {
+    *reinterpret_cast<float4*>(p) = lo;
+    *reinterpret_cast<float4*>(p + 4) = hi;
+  }
+  __device__ double get(int i) const {
+    return static_cast<double>(i < 4 ? (&lo.x)[i] : (&hi.x)[i - 4]);
+  }
+  __device__ void set_pair(int p, double re, double im) {
+    float* dst = p < 2 ? &lo.x + 2 * p : &hi.x + 2 * (p - 2);
+    dst[0] = static_cast<float>(re);
+    dst[1] = static_cast<float>(im);
+  }
+};
+
+// (a + bi)(c + di) with every product and sum rounded separately, as the
+// reference's complex128 multiply on the CPU does.
+template <typename T>
+__device__ __forceinline__ Vec8<T> rotate(const Vec8<T>& x, const double2 (&cs)[4]) {
+#pragma clang fp contract(off)
+  Vec8<T> y;
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const double a = x.get(2 * p), b = x.get(2 * p + 1);
+    const double ac = a * cs[p].x;
+    const double bd = b * cs[p].y;
+    const double ad = a * cs[p].y;
+    const double bc = b * cs[p].x;
+    y.set_pair(p, ac - bd, ad + bc);
+  }
+  return y;
+}
+
+template <typename T, bool kWithQ>
+__global__ __launch_bounds__(kLanesPerRow * kTokensPerBlock)
+void kv_append_rope_kernel(const AppendKernelArgs a) {
+  const int lane = threadIdx.x & (kLanesPerRow - 1);
+  const int tok = blockIdx.x * kTokensPerBlock + (threadIdx.x >> 4);
+  const int row = blockIdx.z;
+  const int head0 = blockIdx.y * kHeadsPerThread;
+
+  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+    if (a.global_end) a.global_end[row] = a.new_global[row];
+    if (a.local_end) a.local_end[row] = a.new_local[row];
+  }
+  if (tok >= a.tokens) return;
+
+  const int fi = tok / a.frame_tokens;
+  const int rem = tok - fi * a.frame_tokens;
+  const int hi = rem / a.grid_w;
+  const int wi = rem - hi * a.grid_w;
+  const int64_t frame = a.start_frame[row] + fi;
+
+  double2 cs[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int p = lane * 4 + j;
+    const int64_t pos = p < a.split_t ? frame : (p < a.split_h ? hi : wi);
+    cs[j] = a.freqs[pos * a.pairs + p];
+  }
+
+  const int64_t e0 = lane * 8;
+  const int64_t dst_tok = a.dst_start[row] + tok;
+  const T* qi = static_cast<const T*>(a.q_in) + row * a.q_in_st.row + tok * a.q_in_st.token + e0;
+  const T* ki = static_cast<const T*>(a.k_in) + row * a.k_in_st.row + tok * a.k_in_st.token + e0;
+  const T* vi = static_cast<const T*>(a.v_in) + row * a.v_in_st.row + tok * a.v_in_st.token + e0;
+  T* qo = static_cast<T*>(a.q_out) + row * a.q_out_st.row + tok * a.q_out_st.token + e0;
+  T* kc = static_cast<T*>(a.k_cache) + row * a.k_st.row + dst_tok * a.k_st.token + e0;
+  T* vc = static_cast<T*>(a.v_cache) + row * a.v_st.row + dst_tok * a.v_st.token + e0;
+
+  Vec8<T> q[kHeadsPerThread], k[kHeadsPerThread], v[kHeadsPerThread];
+#pragma unroll
+  for (int j = 0; j < kHeadsPerThread; ++j) {
+    const int h = head0 + j;
+    if (h < a.heads) {
+      k[j] = Vec8<T>::load(ki + h * a.k_in_st.head);
+      v[j] = Vec8<T>::load(vi + h * a.v_in_st.head);
+      if (kWithQ) q[j] = Vec8<T>::load(qi + h * a.q_in_st.head);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < kHeadsPerThread; ++j) {
+    const int h = head0 + j;
+    if (h < a.heads) {
+      v[j].store(vc + h * a.v_st.head);
+      rotate(k[j], cs).store(kc + h * a.k_st.head);
+      if (kWithQ) rotate(q[j], cs).store(qo + h * a.q_out_st.head);
+    }
+  }
+}
+
+bool stride_ok(const sdv2_stride3& s, int vec) {
+  return s.row % vec == 0 && s.token % vec == 0 && s.head % vec == 0;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace
+
+extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
+  if (!p) return SDV2_ERR_INVALID_ARG;
+  if (p->head_dim != SDV2_HEAD_DIM) return SDV2_ERR_UNSUPPORTED;
+  if (p->dtype != SDV2_BF16 && p->dtype != SDV2_F32) return SDV2_ERR_UNSUPPORTED;
+  if (p->rows < 0 || p->tokens < 0 || p->heads <= 0) return SDV2_ERR_INVALID_ARG;
+  if (p->rows > SDV2_MAX_ROWS) return SDV2_ERR_INVALID_ARG;
+  if (p->rows == 0 || p->tokens == 0) return SDV2_OK;
+  if (p->grid_f <= 0 || p->grid_h <= 0 || p->grid_w <= 0) return SDV2_ERR_INVALID_ARG;
+  if (static_cast<int64_t>(p->grid_f) * p->grid_h * p->grid_w != p->tokens) return SDV2_ERR_INVALID_ARG;
+  if (!p->k_in || !p->v_in || !p->k_cache || !p->v_cache || !p->freqs) return SDV2_ERR_INVALID_ARG;
+  if ((p->q_in == nullptr) != (p->q_out == nullptr)) return SDV2_ERR_INVALID_ARG;
+  if (!p->start_frame || !p->dst_start) return SDV2_ERR_INVALID_ARG;
+  if ((p->global_end_index || p->local_end_index) && (!p->new_global_end || !p->new_local_end))
+    return SDV2_ERR_INVALID_ARG;
+  const bool with_q = p->q_in != nullptr;
+
+  // 16-byte vector access: 8 bf16 or 4 floats per transaction.
+  const int vec = p->dtype == SDV2_BF16 ? 8 : 4;
+  const void* ptrs[] = {p->q_in, p->k_in, p->v_in, p->q_out, p->k_cache, p->v_cache};
+  for (const void* ptr : ptrs)
+    if (ptr && !aligned16(ptr)) return SDV2_ERR_INVALID_ARG;
+  if (!stride_ok(p->k_in_stride, vec) || !stride_ok(p->v_in_stride, vec) ||
+      !stride_ok(p->k_cache_stride, vec) || !stride_ok(p->v_cache_stride, vec))
+    return SDV2_ERR_INVALID_ARG;
+  if (with_q && (!stride_ok(p->q_in_stride, vec) || !stride_ok(p->q_out_stride, vec)))
+    return SDV2_ERR_INVALID_ARG;
+
+  if (p->grid_h > p->freq_rows || p->grid_w > p->freq_rows) return SDV2_ERR_OUT_OF_RANGE;
+  for (int i = 0; i < p->rows; ++i) {
+    if (p->start_frame[i] < 0 || p->start_frame[i] + p->grid_f > p->freq_rows) return SDV2_ERR_OUT_OF_RANGE;
+    if (p->dst_start[i] < 0 || p->dst_start[i] + p->tokens > p->cache_tokens) return SDV2_ERR_OUT_OF_RANGE;
+  }
+
+  AppendKernelArgs a{};
+  a.q_in = p->q_in; a.k_in = p->k_in; a.v_in = p->v_in;
+  a.q_out = p->q_out; a.k_cache = p->k_cache; a.v_cache = p->v_cache;
+  a.q_in_st = p->q_in_stride; a.k_in_st = p->k_in_stride; a.v_in_st = p->v_in_stride;
+  a.q_out_st = p->q_out_stride; a.k_st = p->k_cache_stride; a.v_st = p->v_cache_stride;
+  a.freqs = reinterpret_cast<const double2*>(p->freqs);
+  a.global_end = p->global_end_index;
+  a.local_end = p->local_end_index;
+  a.tokens = p->tokens; a.heads = p->heads; a.grid_w = p->grid_w;
+  a.frame_tokens = p->grid_h * p->grid_w;
+  a.pairs = p->head_dim / 2;
+  // column split of the table: c - 2*(c/3) | c/3 | c/3  (causal_model.py:77-78)
+  const int third = a.pairs / 3;
+  a.split_t = a.pairs - 2 * third;
+  a.split_h = a.split_t + third;
+  for (int i = 0; i < p->rows; ++i) {
+    a.start_frame[i] = p->start_frame[i];
+    a.dst_start[i] = p->dst_start[i];
+    a.new_global[i] = p->new_global_end ? p->new_global_end[i] : 0;
+    a.new_local[i] = p->new_local_end ? p->new_local_end[i] : 0;
+  }
+
+  dim3 block(kLanesPerRow * kTokensPerBlock);
+  dim3 grid((p->tokens + kTokensPerBlock - 1) / kTokensPerBlock,
+            (p->heads + kHeadsPerThread - 1) / kHeadsPerThread, p->rows);
+  hipStream_t stream = static_cast<hipStream_t>(p->stream);
+  if (p->dtype == SDV2_BF16) {
+    if (with_q) hipLaunchKernelGGL((kv_append_rope_kernel<uint16_t, true>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((kv_append_rope_kernel<uint16_t, false>), grid, block, 0, stream, a);
+  } else {
+    if (with_q) hipLaunchKernelGGL((kv_append_rope_kernel<float, true>), grid, block, 0, stream, a);
+    else hipLaunchKernelGGL((kv_append_rope_kernel<float, false>), grid, block, 0, stream, a);
+  }
+  return hipGetLastError() == hipSuccess ? SDV2_OK : SDV2_ERR_LAUNCH;
+}

@@ -1,0 +1,41 @@
+// Small entry points of the sdv2kv C ABI that are not kernels of the path
+// itself: version, status strings and the counter-calibration copy.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "sdv2kv.h"
+
+namespace {
+
+__global__ __launch_bounds__(256) void copy16_kernel(uint4* dst, const uint4* src, size_t n16) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
+}  // namespace
+
+extern "C" int sdv2_abi_version(void) { return SDV2KV_ABI_VERSION; }
+
+extern "C" const char* sdv2_status_string(int status) {
+  switch (status) {
+    case SDV2_OK: return "ok";
+    case SDV2_ERR_INVALID_ARG: return "invalid argument (null pointer, bad shape, misaligned pointer or stride)";
+    case SDV2_ERR_UNSUPPORTED: return "unsupported head_dim or dtype";
+    case SDV2_ERR_OUT_OF_RANGE: return "write range outside the cache or RoPE position beyond the table";
+    case SDV2_ERR_WORKSPACE: return "split-KV workspace missing or too small";
+    case SDV2_ERR_LAUNCH: return "kernel launch failed";
+    default: return "unknown status";
+  }
+}
+
+extern "C" int sdv2_copy_bytes(void* dst, const void* src, size_t bytes, void* stream) {
+  if (bytes == 0) return SDV2_OK;
+  if (!dst || !src) return SDV2_ERR_INVALID_ARG;
+  if ((reinterpret_cast<uintptr_t>(dst) | reinterpret_cast<uintptr_t>(src) | bytes) & 15) return SDV2_ERR_INVALID_ARG;
+  const size_t n16 = bytes / 16;
+  size_t blocks = (n16 + 255) / 256;
+  if (blocks > 256 * 32) blocks = 256 * 32;
+  hipLaunchKernelGGL(copy16_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<uint4*>(dst), static_cast<const uint4*>(src), n16);
+  return hipGetLastError() == hipSuccess ? SDV2_OK : SDV2_ERR_LAUNCH;
+}

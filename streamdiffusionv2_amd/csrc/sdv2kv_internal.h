@@ -1,0 +1,23 @@
+// Device helpers shared by the sdv2kv kernels (gfx950 only).
+#ifndef SDV2KV_INTERNAL_H
+#define SDV2KV_INTERNAL_H
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sdv2 {
+
+// float -> bfloat16 bit pattern, round-to-nearest-even, NaN -> 0x7FC0: the
+// rounding PyTorch applies when a float (or a double already narrowed to
+// float) is stored as bfloat16.
+__device__ __forceinline__ uint32_t f32_to_bf16_rne(float f) {
+  const uint32_t u = __float_as_uint(f);
+  if (f != f) return 0x7fc0u;
+  return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+
+}  // namespace sdv2
+
+#endif  // SDV2KV_INTERNAL_H

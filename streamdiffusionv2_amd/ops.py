@@ -1,0 +1,241 @@
+"""Operator-level Python surface over the sdv2kv C ABI.
+
+``flash_attn_with_kvcache`` keeps the four-argument call the reference makes
+(models/wan/causal_model.py:353-358); ``kv_append_rope`` is the fused
+replacement for causal_rope_apply + the per-row slice writes (:253-266,
+:321-342).  PyTorch supplies device memory and the current stream only.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from . import _capi
+
+HEAD_DIM = _capi.HEAD_DIM
+
+_DTYPES = {torch.bfloat16: _capi.DTYPE_BF16, torch.float32: _capi.DTYPE_F32}
+
+
+def _require_gpu(*tensors: torch.Tensor) -> torch.device:
+    dev = tensors[0].device
+    for t in tensors:
+        if t is None:
+            continue
+        if t.device.type != "cuda":
+            raise RuntimeError(
+                "sdv2kv operators run on the GPU only (tensor on %s); there is no CPU path" % t.device
+            )
+        if t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {t.device} vs {dev}")
+    return dev
+
+
+def _stride3(t: torch.Tensor, name: str) -> _capi.Stride3:
+    if t.dim() != 4 or t.shape[-1] != HEAD_DIM:
+        raise RuntimeError(f"{name}: expected [rows, tokens, heads, {HEAD_DIM}], got {tuple(t.shape)}")
+    if t.shape[-1] > 1 and t.stride(-1) != 1:
+        raise RuntimeError(f"{name}: last dimension must be contiguous (stride {t.stride(-1)})")
+    return _capi.Stride3(t.stride(0), t.stride(1), t.stride(2))
+
+
+def _stream_ptr(dev: torch.device) -> int:
+    return torch.cuda.current_stream(dev).cuda_stream
+
+
+def _i64_array(values: Sequence[int]):
+    return (C.c_int64 * len(values))(*[int(v) for v in values])
+
+
+_FREQS_CACHE: dict = {}
+
+
+def device_freqs(freqs: torch.Tensor, device: torch.device) -> torch.Tensor:
+    """The complex128 [rows, 64] RoPE table as float64 [rows, 64, 2] on
+    ``device``.  Converted once per (table, device)."""
+    key = (id(freqs), freqs._version, freqs.data_ptr(), str(device))
+    hit = _FREQS_CACHE.get(key)
+    if hit is not None and hit[0] is freqs:
+        return hit[1]
+    if freqs.dtype != torch.complex128 or freqs.dim() != 2 or freqs.shape[1] != HEAD_DIM // 2:
+        raise RuntimeError(
+            f"freqs must be complex128 [rows, {HEAD_DIM // 2}], got {freqs.dtype} {tuple(freqs.shape)}"
+        )
+    table = torch.view_as_real(freqs.detach().resolve_conj()).contiguous().to(device)
+    if len(_FREQS_CACHE) > 8:
+        _FREQS_CACHE.clear()
+    _FREQS_CACHE[key] = (freqs, table)
+    return table
+
+
+def kv_append_rope(
+    q: Optional[torch.Tensor],
+    k: torch.Tensor,
+    v: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    freqs_table: torch.Tensor,
+    grid: Tuple[int, int, int],
+    start_frames: Sequence[int],
+    dst_starts: Sequence[int],
+    q_out: Optional[torch.Tensor] = None,
+    global_end_index: Optional[torch.Tensor] = None,
+    local_end_index: Optional[torch.Tensor] = None,
+    new_global_end: Optional[Sequence[int]] = None,
+    new_local_end: Optional[Sequence[int]] = None,
+) -> Optional[torch.Tensor]:
+    """RoPE q and k, write k' and v into the cache at ``dst_starts`` and store
+    the new end indices.  Returns the roped query (``q_out`` or a new tensor).
+
+    ``freqs_table`` is :func:`device_freqs` output.  Rows are processed in
+    groups of at most 16 per launch.
+    """
+    dev = _require_gpu(k, v, k_cache, v_cache, freqs_table, q, q_out, global_end_index, local_end_index)
+    if k.dtype not in _DTYPES:
+        raise RuntimeError(f"unsupported dtype {k.dtype}")
+    for t in (q, v, k_cache, v_cache, q_out):
+        if t is not None and t.dtype != k.dtype:
+            raise RuntimeError(f"dtype mismatch: {t.dtype} vs {k.dtype}")
+    rows, tokens, heads, _ = k.shape
+    if q is not None and q_out is None:
+        q_out = torch.empty((rows, tokens, heads, HEAD_DIM), dtype=q.dtype, device=dev)
+    for name, t in (("q", q), ("v", v), ("q_out", q_out)):
+        if t is not None and tuple(t.shape) != tuple(k.shape):
+            raise RuntimeError(f"{name} shape {tuple(t.shape)} differs from k {tuple(k.shape)}")
+    if k_cache.shape[0] < rows or v_cache.shape != k_cache.shape or k_cache.shape[2] != heads:
+        raise RuntimeError(f"cache shape {tuple(k_cache.shape)} / {tuple(v_cache.shape)} does not fit k {tuple(k.shape)}")
+    if len(start_frames) != rows or len(dst_starts) != rows:
+        raise RuntimeError("start_frames and dst_starts need one entry per row")
+    for idx in (global_end_index, local_end_index):
+        if idx is not None and (idx.dtype != torch.int64 or idx.numel() < rows or not idx.is_contiguous()):
+            raise RuntimeError("end-index tensors must be contiguous int64 with one entry per row")
+    if freqs_table.dtype != torch.float64 or not freqs_table.is_contiguous():
+        raise RuntimeError("freqs_table must be the contiguous float64 view from device_freqs()")
+
+    lib = _capi.lib()
+    stream = _stream_ptr(dev)
+    with torch.cuda.device(dev):
+        for r0 in range(0, rows, _capi.MAX_ROWS):
+            r1 = min(rows, r0 + _capi.MAX_ROWS)
+            p = _capi.AppendParams()
+            sl = slice(r0, r1)
+            if q is not None:
+                p.q_in, p.q_in_stride = q[sl].data_ptr(), _stride3(q, "q")
+                p.q_out, p.q_out_stride = q_out[sl].data_ptr(), _stride3(q_out, "q_out")
+            p.k_in, p.k_in_stride = k[sl].data_ptr(), _stride3(k, "k")
+            p.v_in, p.v_in_stride = v[sl].data_ptr(), _stride3(v, "v")
+            p.k_cache, p.k_cache_stride = k_cache[sl].data_ptr(), _stride3(k_cache, "k_cache")
+            p.v_cache, p.v_cache_stride = v_cache[sl].data_ptr(), _stride3(v_cache, "v_cache")
+            p.freqs = freqs_table.data_ptr()
+            p.freq_rows = freqs_table.shape[0]
+            p.dtype = _DTYPES[k.dtype]
+            p.rows, p.tokens, p.heads, p.head_dim = r1 - r0, tokens, heads, HEAD_DIM
+            p.grid_f, p.grid_h, p.grid_w = (int(x) for x in grid)
+            p.cache_tokens = k_cache.shape[1]
+            sf = _i64_array(start_frames[r0:r1])
+            ds = _i64_array(dst_starts[r0:r1])
+            p.start_frame = C.cast(sf, C.POINTER(C.c_int64))
+            p.dst_start = C.cast(ds, C.POINTER(C.c_int64))
+            if global_end_index is not None or local_end_index is not None:
+                if new_global_end is None or new_local_end is None:
+                    raise RuntimeError("new_global_end/new_local_end are required with the index tensors")
+                ng = _i64_array(new_global_end[r0:r1])
+                nl = _i64_array(new_local_end[r0:r1])
+                p.new_global_end = C.cast(ng, C.POINTER(C.c_int64))
+                p.new_local_end = C.cast(nl, C.POINTER(C.c_int64))
+                if global_end_index is not None:
+                    p.global_end_index = global_end_index.data_ptr() + 8 * r0
+                if local_end_index is not None:
+                    p.local_end_index = local_end_index.data_ptr() + 8 * r0
+            p.stream = stream
+            _capi.check(lib.sdv2_kv_append_rope(C.byref(p)), "sdv2_kv_append_rope")
+    return q_out
+
+
+_WORKSPACES: dict = {}
+
+
+def _workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
+    """Per-device scratch for split-KV partials, grown on demand and reused
+    (stream-ordered reuse is safe: merge always follows its split kernel)."""
+    ws = _WORKSPACES.get(dev)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=dev)
+        _WORKSPACES[dev] = ws
+    return ws
+
+
+def swa_attention(
+    q: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    seq_lens: Optional[torch.Tensor] = None,
+    out: Optional[torch.Tensor] = None,
+    num_splits: int = 0,
+    softmax_scale: Optional[float] = None,
+    workspace: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """out[b] = softmax(q[b] k_cache[b,:seq_lens[b]]^T * scale) v_cache[b,:seq_lens[b]].
+
+    q [B,S,H,128] bf16; k_cache/v_cache [B,L,H,128] bf16 views with any row /
+    token / head strides; seq_lens int32 [B] on the device (None = L).
+    """
+    dev = _require_gpu(q, k_cache, v_cache, seq_lens, out, workspace)
+    if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
+        raise RuntimeError("swa_attention computes in bf16; got %s/%s/%s" % (q.dtype, k_cache.dtype, v_cache.dtype))
+    rows, q_tokens, heads, _ = q.shape
+    if k_cache.shape[0] != rows or k_cache.shape[2] != heads or v_cache.shape != k_cache.shape:
+        raise RuntimeError(f"cache view {tuple(k_cache.shape)} / {tuple(v_cache.shape)} does not match q {tuple(q.shape)}")
+    if seq_lens is not None and (seq_lens.dtype != torch.int32 or seq_lens.numel() != rows or not seq_lens.is_contiguous()):
+        raise RuntimeError("seq_lens must be a contiguous int32 tensor with one entry per row")
+    if out is None:
+        out = torch.empty((rows, q_tokens, heads, HEAD_DIM), dtype=torch.bfloat16, device=dev)
+    elif out.dtype != torch.bfloat16 or tuple(out.shape) != tuple(q.shape):
+        raise RuntimeError("out must be bf16 with q's shape")
+
+    lib = _capi.lib()
+    max_seq_len = k_cache.shape[1]
+    if num_splits <= 0:
+        num_splits = lib.sdv2_swa_attn_default_splits(rows, q_tokens, heads, max_seq_len)
+    need = lib.sdv2_swa_attn_workspace_bytes(rows, q_tokens, heads, max_seq_len, num_splits)
+    if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
+        workspace = _workspace(dev, need)
+
+    p = _capi.AttnParams()
+    p.q, p.q_stride = q.data_ptr(), _stride3(q, "q")
+    p.k_cache, p.k_stride = k_cache.data_ptr(), _stride3(k_cache, "k_cache")
+    p.v_cache, p.v_stride = v_cache.data_ptr(), _stride3(v_cache, "v_cache")
+    p.out, p.out_stride = out.data_ptr(), _stride3(out, "out")
+    p.seq_lens = seq_lens.data_ptr() if seq_lens is not None else None
+    p.rows, p.q_tokens, p.heads, p.head_dim = rows, q_tokens, heads, HEAD_DIM
+    p.max_seq_len = max_seq_len
+    p.num_splits = num_splits
+    p.softmax_scale = float(softmax_scale) if softmax_scale else 0.0
+    if need:
+        p.workspace = workspace.data_ptr()
+        p.workspace_bytes = workspace.numel() * workspace.element_size()
+    p.stream = _stream_ptr(dev)
+    with torch.cuda.device(dev):
+        _capi.check(lib.sdv2_swa_attn_fwd(C.byref(p)), "sdv2_swa_attn_fwd")
+    return out
+
+
+def flash_attn_with_kvcache(q, k_cache, v_cache, cache_seqlens=None):
+    """Same call as the reference makes on flash_attn_interface
+    (causal_model.py:353-358): defaults mean causal=False and scale 1/sqrt(D)."""
+    if cache_seqlens is not None and cache_seqlens.dtype != torch.int32:
+        cache_seqlens = cache_seqlens.to(torch.int32)
+    return swa_attention(q, k_cache, v_cache, cache_seqlens)
+
+
+def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
+    """Plain 16-byte-vector copy with the library's own kernel (used to scale
+    hardware counters against a transfer of known size)."""
+    dev = _require_gpu(dst, src)
+    n = src.numel() * src.element_size()
+    if dst.numel() * dst.element_size() != n or not dst.is_contiguous() or not src.is_contiguous():
+        raise RuntimeError("copy_bytes needs contiguous tensors of equal byte size")
+    with torch.cuda.device(dev):
+        _capi.check(_capi.lib().sdv2_copy_bytes(dst.data_ptr(), src.data_ptr(), n, _stream_ptr(dev)), "sdv2_copy_bytes")

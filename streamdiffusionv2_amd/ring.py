@@ -1,0 +1,181 @@
+"""Host side of the ring KV cache: the per-layer ``kv_cache`` dict and the
+integer state machine that decides where each chunk lands.
+
+The dict keeps the reference's contract (models/wan/causal_stream_inference.py:98-105):
+``k``/``v`` of logical shape [B, cap, H, 128], ``global_end_index`` and
+``local_end_index`` as int64 [B] device tensors mutated in place, and the
+python ints ``total_steps``/``current_step``.  ``k``/``v`` are permuted views of
+head-major [B, H, cap, 128] buffers, so a chunk's rows for one head are one
+contiguous run in HBM.
+
+The placement policy restates models/wan/causal_model.py:268-342 on host
+integers only.  The reference reads the two index tensors back with ``.item()``
+for every row of every layer; here the host carries a mirror of them (they are
+a pure function of the host-known ``current_start`` sequence), validated
+against the tensors' identity and version counter, so the steady state issues
+no device-to-host copy at all.  The kernel stores the new index values, which
+keeps the tensors authoritative for every external consumer of the dict.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional, Sequence
+
+import torch
+
+HEAD_DIM = 128
+_MIRROR_KEY = "_sdv2_host_index_mirror"
+
+
+def new_kv_cache(
+    num_layers: int,
+    batch_size: int,
+    cache_tokens: int,
+    num_heads: int,
+    total_steps: int,
+    dtype: torch.dtype = torch.bfloat16,
+    device="cuda",
+    head_major: bool = True,
+) -> List[dict]:
+    """Allocate the per-layer cache dicts of
+    ``CausalStreamInferencePipeline._initialize_kv_cache``
+    (causal_stream_inference.py:87-107)."""
+    layers = []
+    for _ in range(num_layers):
+        if head_major:
+            k = torch.zeros([batch_size, num_heads, cache_tokens, HEAD_DIM], dtype=dtype, device=device).permute(0, 2, 1, 3)
+            v = torch.zeros([batch_size, num_heads, cache_tokens, HEAD_DIM], dtype=dtype, device=device).permute(0, 2, 1, 3)
+        else:
+            k = torch.zeros([batch_size, cache_tokens, num_heads, HEAD_DIM], dtype=dtype, device=device)
+            v = torch.zeros([batch_size, cache_tokens, num_heads, HEAD_DIM], dtype=dtype, device=device)
+        layers.append(
+            {
+                "k": k,
+                "v": v,
+                "global_end_index": torch.tensor([0], dtype=torch.long, device=device),
+                "local_end_index": torch.tensor([0], dtype=torch.long, device=device),
+                "total_steps": total_steps,
+                "current_step": total_steps,
+            }
+        )
+    return layers
+
+
+def replicate_for_stream_batch(kv_cache: List[dict], batch_size: int) -> None:
+    """One cache per denoising stage (causal_stream_inference.py:221-225).
+    ``repeat`` on the underlying head-major buffer keeps the layout."""
+    for entry in kv_cache:
+        for name in ("k", "v"):
+            t = entry[name]
+            if t.stride(2) > t.stride(1):  # head-major view [B, cap, H, D]
+                entry[name] = t.permute(0, 2, 1, 3).repeat(batch_size, 1, 1, 1).permute(0, 2, 1, 3)
+            else:
+                entry[name] = t.repeat(batch_size, 1, 1, 1)
+        entry["global_end_index"] = entry["global_end_index"].repeat(batch_size)
+        entry["local_end_index"] = entry["local_end_index"].repeat(batch_size)
+        entry.pop(_MIRROR_KEY, None)
+
+
+@dataclass
+class _IndexMirror:
+    g_tensor: torch.Tensor
+    l_tensor: torch.Tensor
+    g_version: int
+    l_version: int
+    global_end: List[int]
+    local_end: List[int]
+
+    def valid_for(self, kv_cache: dict) -> bool:
+        g, l = kv_cache["global_end_index"], kv_cache["local_end_index"]
+        return (
+            g is self.g_tensor and l is self.l_tensor
+            and g._version == self.g_version and l._version == self.l_version
+        )
+
+
+def _mirror(kv_cache: dict) -> _IndexMirror:
+    m: Optional[_IndexMirror] = kv_cache.get(_MIRROR_KEY)
+    if m is None or not m.valid_for(kv_cache):
+        g, l = kv_cache["global_end_index"], kv_cache["local_end_index"]
+        m = _IndexMirror(g, l, g._version, l._version, [int(x) for x in g.tolist()], [int(x) for x in l.tolist()])
+        kv_cache[_MIRROR_KEY] = m
+    return m
+
+
+@dataclass
+class AppendPlan:
+    """What one layer call does, row by row."""
+    dst_start: List[int]      # first cache token written
+    new_global_end: List[int]
+    new_local_end: List[int]  # == seq_lens of the attention that follows
+
+    @property
+    def max_seq_len(self) -> int:
+        return max(self.new_local_end)
+
+
+def plan_append(
+    kv_cache: dict,
+    evict_idx: List[List[int]],
+    current_start: Sequence[int],
+    n_new: int,
+    frame_tokens: int,
+    sink_size: int,
+) -> AppendPlan:
+    """Advance the ring state by one call and say where the chunk of each row
+    goes.  Mutates ``evict_idx`` and ``kv_cache['current_step']`` and the host
+    index mirror exactly as causal_model.py:279-342 mutates its state; the
+    device index tensors are written by the append kernel.
+
+    Raises IndexError when the cache is full and the eviction queue is empty
+    (causal_model.py:306) and ValueError when the slot would start before the
+    cache (the reference's negative slice would fail on a shape mismatch).
+    """
+    cap = kv_cache["k"].shape[1]
+    cache_rows = kv_cache["k"].shape[0]
+    sink_tokens = sink_size * frame_tokens
+    m = _mirror(kv_cache)
+    if len(m.local_end) < len(current_start):
+        raise ValueError(
+            f"current_start has {len(current_start)} rows but the cache indices have {len(m.local_end)}"
+        )
+
+    dst_start, new_g, new_l = [], [], []
+    for i, c_start in enumerate(current_start):
+        c_start = int(c_start)
+        c_end = c_start + n_new
+        queue = evict_idx[i]
+        if c_end > cap or m.local_end[i] >= cap:
+            m.global_end[i], m.local_end[i] = c_start, cap
+            dst_end = queue[0]
+            if cache_rows == 1 and kv_cache["current_step"] > 1:
+                kv_cache["current_step"] -= 1
+            else:
+                head = queue.pop(0)
+                if head > sink_tokens:
+                    queue.append(head)
+                kv_cache["current_step"] = kv_cache["total_steps"]
+            local_new = cap
+        else:
+            local_new = m.local_end[i] + c_end - m.global_end[i]
+            next_end = c_end + n_new
+            if sink_tokens < next_end <= cap and (not queue or queue[-1] != next_end):
+                queue.append(next_end)
+            dst_end = local_new
+        start = dst_end - n_new
+        if start < 0 or dst_end > cap:
+            raise ValueError(f"row {i}: chunk of {n_new} tokens would be written at [{start}, {dst_end}) of a {cap}-token cache")
+        dst_start.append(start)
+        new_g.append(c_end)
+        new_l.append(local_new)
+        m.global_end[i], m.local_end[i] = c_end, local_new
+    return AppendPlan(dst_start, new_g, new_l)
+
+
+def closed_form_slot(chunk: int, n_slots: int, n_permanent: int) -> int:
+    """Slot of chunk number ``chunk`` for uniform chunks that divide the
+    cache, one pass per chunk and no adaptive refresh: fill 0..n_slots-1, then
+    rotate over the evictable slots.  Eviction is therefore an index update."""
+    if chunk < n_slots:
+        return chunk
+    return n_permanent + (chunk - n_slots) % (n_slots - n_permanent)

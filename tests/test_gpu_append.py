@@ -1,0 +1,60 @@
+"""GPU parity of the fused RoPE-on-write append against the CPU oracle:
+cache contents, roped query and indices must be bit-exact."""
+import pytest
+import torch
+
+from oracle import sdv2_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+
+def _bits(t):
+    return t.contiguous().view(torch.int16 if t.dtype == torch.bfloat16 else torch.int32)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("head_major", [True, False])
+@pytest.mark.parametrize("grid,heads,rows", [((1, 6, 10), 12, 1), ((3, 5, 8), 5, 3), ((2, 30, 52), 12, 2)])
+def test_append_matches_oracle_bitwise(gpu_device, dtype, head_major, grid, heads, rows):
+    from streamdiffusionv2_amd import ops
+
+    torch.manual_seed(1234)
+    f, h, w = grid
+    S = f * h * w
+    cap = 4 * S
+    freqs = oracle.build_freqs()
+    q = torch.randn(rows, S, heads, 128).to(dtype)
+    k = torch.randn(rows, S, heads, 128).to(dtype)
+    v = torch.randn(rows, S, heads, 128).to(dtype)
+    start_frames = [7 + 3 * r for r in range(rows)]
+    dst = [(r % 4) * S for r in range(rows)]
+
+    want_q = oracle.causal_rope_apply(q, [grid] * rows, freqs, start_frames)
+    want_k = oracle.causal_rope_apply(k, [grid] * rows, freqs, start_frames)
+
+    if head_major:
+        kc = torch.zeros(rows, heads, cap, 128, dtype=dtype, device=gpu_device).permute(0, 2, 1, 3)
+        vc = torch.zeros(rows, heads, cap, 128, dtype=dtype, device=gpu_device).permute(0, 2, 1, 3)
+    else:
+        kc = torch.zeros(rows, cap, heads, 128, dtype=dtype, device=gpu_device)
+        vc = torch.zeros(rows, cap, heads, 128, dtype=dtype, device=gpu_device)
+    g_idx = torch.zeros(rows, dtype=torch.long, device=gpu_device)
+    l_idx = torch.zeros(rows, dtype=torch.long, device=gpu_device)
+    table = ops.device_freqs(freqs, gpu_device)
+    got_q = ops.kv_append_rope(
+        q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), kc, vc, table, grid, start_frames, dst,
+        global_end_index=g_idx, local_end_index=l_idx,
+        new_global_end=[100 + r for r in range(rows)], new_local_end=[200 + r for r in range(rows)],
+    )
+    torch.cuda.synchronize()
+    assert torch.equal(_bits(got_q.cpu()), _bits(want_q))
+    kc_cpu, vc_cpu = kc.cpu(), vc.cpu()
+    for r in range(rows):
+        assert torch.equal(_bits(kc_cpu[r, dst[r]:dst[r] + S]), _bits(want_k[r]))
+        assert torch.equal(_bits(vc_cpu[r, dst[r]:dst[r] + S]), _bits(v[r]))
+        # everything outside the written slot stays zero
+        mask = torch.ones(cap, dtype=torch.bool)
+        mask[dst[r]:dst[r] + S] = False
+        assert not kc_cpu[r, mask].any() and not vc_cpu[r, mask].any()
+    assert g_idx.tolist() == [100 + r for r in range(rows)]
+    assert l_idx.tolist() == [200 + r for r in range(rows)]
