@@ -1,0 +1,262 @@
+#!/usr/bin/env python3
+"""Benchmark of the ring KV-cache path on one MI355X.
+
+One step = one chunk through every layer's (RoPE-on-write append + sink/window
+attention), inputs already resident in HBM, steady state (cache full, ring
+rotating).  Prints ONE JSON line: whole-job tokens/s, per-chunk latency, the
+roofline of the dominant kernel (timed live with HIP events on the launch
+stream) and the CPU oracle timed on the host cores of the same box.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload 2]
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", type=int, default=2, help="index into BASELINE.json configs (1-based)")
+    ap.add_argument("--num-splits", type=int, default=0)
+    ap.add_argument("--skip-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-chunks", type=int, default=2, help="steady-state chunks timed on the CPU oracle")
+    ap.add_argument("--cpu-layers", type=int, default=1)
+    return ap.parse_args()
+
+
+def build_freqs():
+    """The model's RoPE table, built on the CPU in float64 as the reference
+    model does at construction (causal_model.py:631-638)."""
+    from streamdiffusionv2_amd.rope import build_freqs as _bf
+
+    return _bf()
+
+
+def gpu_bench(args, w):
+    from streamdiffusionv2_amd import _capi, ops, ring, workloads
+    from streamdiffusionv2_amd.attention import RingKVPath
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    freqs = build_freqs()
+    S, H, B = w.chunk_tokens, w.heads, w.rows
+    grid_sizes = torch.tensor([list(w.grid)] * B, dtype=torch.long)
+    caches = ring.new_kv_cache(w.layers, 1, w.cache_tokens, H, total_steps=1, dtype=w.dtype, device=dev)
+    if B > 1:
+        ring.replicate_for_stream_batch(caches, B)
+    paths = [RingKVPath(sink_size=w.sink_size, adapt_sink_thr=-1) for _ in range(w.layers)]
+    # per-layer inputs, resident in HBM before the clock starts
+    qkv = []
+    for layer in range(w.layers):
+        q, k, v = workloads.make_qkv(w, 0, layer)
+        qkv.append((q.to(dev), k.to(dev), v.to(dev)))
+    max_chunk = (1024 - w.grid[0]) // w.grid[0]     # keep the frame index inside the RoPE table
+    state = {"call": 0}
+
+    def step(timers=None):
+        call = state["call"]
+        starts = [min(c, max_chunk) * S for c in workloads.row_chunks(w, call)]
+        for layer in range(w.layers):
+            q, k, v = qkv[layer]
+            if timers is None:
+                paths[layer].attend(q, k, v, grid_sizes, freqs, caches[layer], starts)
+            else:
+                timed_layer(paths[layer], q, k, v, caches[layer], starts, timers)
+        state["call"] += 1
+
+    table = ops.device_freqs(freqs, dev)
+
+    def timed_layer(path, q, k, v, cache, starts, timers):
+        """Same launches as attend(), with HIP events between the kernels."""
+        frame_tokens = w.frame_tokens
+        if path.evict_idx is None:
+            path.evict_idx = [[]]
+        if len(path.evict_idx) < B:
+            path.evict_idx = [list(path.evict_idx[0]) for _ in range(B)]
+        plan = ring.plan_append(cache, path.evict_idx, starts, S, frame_tokens, path.sink_size)
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+        ev[0].record()
+        roped_q = ops.kv_append_rope(
+            q, k, v, cache["k"], cache["v"], table, w.grid, [c // frame_tokens for c in starts], plan.dst_start,
+            global_end_index=cache["global_end_index"], local_end_index=cache["local_end_index"],
+            new_global_end=plan.new_global_end, new_local_end=plan.new_local_end)
+        ev[1].record()
+        span = plan.max_seq_len
+        kc, vc = cache["k"][:, :span], cache["v"][:, :span]
+        splits = args.num_splits or _capi.lib().sdv2_swa_attn_default_splits(B, S, H, span)
+        if splits > 1:
+            out = ops.swa_attention(roped_q, kc, vc, None, num_splits=splits, stages=_capi.STAGE_PARTIAL)
+            ev[2].record()
+            ops.swa_attention(roped_q, kc, vc, None, out=out, num_splits=splits, stages=_capi.STAGE_MERGE)
+        else:
+            ops.swa_attention(roped_q, kc, vc, None, num_splits=1)
+            ev[2].record()
+        ev[3].record()
+        timers.append(ev)
+
+    # fill the ring (untimed), then warm up
+    fill_calls = w.cache_tokens // S + B
+    for _ in range(fill_calls + args.warmup):
+        step()
+    torch.cuda.synchronize()
+
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+
+    # instrumented pass over the same steps: per-kernel durations
+    timers = []
+    for _ in range(args.steps):
+        step(timers)
+    torch.cuda.synchronize()
+    t_append = sum(e[0].elapsed_time(e[1]) for e in timers) / len(timers)
+    t_attn = sum(e[1].elapsed_time(e[2]) for e in timers) / len(timers)
+    t_merge = sum(e[2].elapsed_time(e[3]) for e in timers) / len(timers)
+    splits = args.num_splits or _capi.lib().sdv2_swa_attn_default_splits(B, S, H, w.cache_tokens)
+    return {
+        "ms_per_step": ms_per_step,
+        "append_ms": t_append,
+        "attn_ms": t_attn,
+        "merge_ms": t_merge,
+        "splits": splits,
+    }
+
+
+def cpu_baseline(args, w):
+    """The CPU oracle (a PyTorch restatement of the reference's op sequence)
+    on this box's host cores: a bounded sample of steady-state chunks on a few
+    layers, scaled to the full layer count."""
+    from oracle import sdv2_oracle as oracle
+    from streamdiffusionv2_amd import workloads
+
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    freqs = oracle.build_freqs()
+    S, B = w.chunk_tokens, w.rows
+    n_layers = min(args.cpu_layers, w.layers)
+    caches = oracle.new_kv_cache(n_layers, 1, w.cache_tokens, w.heads, 1, dtype=w.dtype)
+    if B > 1:
+        oracle.replicate_for_stream_batch(caches, B)
+    layers = [oracle.RingAttentionOracle(sink_size=w.sink_size, adapt_sink_thr=-1) for _ in range(n_layers)]
+    grids = [list(w.grid)] * B
+    qkv = [workloads.make_qkv(w, 0, layer) for layer in range(n_layers)]
+    fill_calls = w.cache_tokens // S + B
+    call = 0
+    for _ in range(fill_calls):
+        starts = workloads.row_starts(w, call)
+        for layer in range(n_layers):
+            q, k, v = qkv[layer]
+            layers[layer].step(q, k, v, grids, freqs, caches[layer], starts, with_attention=False)
+        call += 1
+    t0 = time.perf_counter()
+    for _ in range(args.cpu_chunks):
+        starts = workloads.row_starts(w, call)
+        for layer in range(n_layers):
+            q, k, v = qkv[layer]
+            layers[layer].step(q, k, v, grids, freqs, caches[layer], starts)
+        call += 1
+    dt = time.perf_counter() - t0
+    per_layer_chunk = dt / (args.cpu_chunks * n_layers)
+    per_chunk = per_layer_chunk * w.layers
+    return {
+        "value": B * S / per_chunk,
+        "unit": "tokens/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": (f"{args.cpu_chunks} steady-state chunks x {n_layers} layer(s) of {w.name} "
+                   f"({dt:.1f} s), scaled to {w.layers} layers; torch {torch.__version__}"),
+        "ms_per_step": per_chunk * 1e3,
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the ring KV-cache path is not sharded across GPUs in this "
+              "build (no collectives); run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+    from streamdiffusionv2_amd import workloads
+
+    w = workloads.WORKLOADS[args.workload]
+    if w.dtype != torch.bfloat16:
+        print("the GPU attention kernel computes in bf16; workload 1 is the CPU-plumbing parity case, "
+              "not a bench line", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (the KV-cache path has no CPU fallback)", file=sys.stderr)
+        sys.exit(2)
+
+    g = gpu_bench(args, w)
+    tokens = w.rows * w.chunk_tokens
+    attn_s = g["attn_ms"] * 1e-3
+    achieved_tflops = w.attn_flops() / attn_s / 1e12
+    append_gbs = w.append_bytes(with_q=True) / (g["append_ms"] * 1e-3) / 1e9
+    result = {
+        "metric": "kv_append_attn_tokens_per_s",
+        "value": tokens / (g["ms_per_step"] * 1e-3),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": g["ms_per_step"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": w.name,
+            "layers": w.layers, "rows": w.rows, "heads": w.heads, "head_dim": 128,
+            "chunk_tokens": w.chunk_tokens, "cache_tokens": w.cache_tokens,
+            "grid": list(w.grid), "kv_splits": g["splits"],
+        },
+        "roofline": {
+            "kernel": "swa_attn_fwd_kernel",
+            "bound": "mfma",
+            "achieved": achieved_tflops,
+            "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": achieved_tflops / PEAK_BF16_TFLOPS,
+            "traffic": None,
+            "flops_per_launch": w.attn_flops(),
+            "avg_launch_ms": g["attn_ms"],
+        },
+        "roofline_append": {
+            "kernel": "kv_append_rope_kernel",
+            "bound": "hbm",
+            "achieved": append_gbs,
+            "peak": PEAK_HBM_GBS,
+            "unit": "GB/s",
+            "frac": append_gbs / PEAK_HBM_GBS,
+            "traffic": None,
+            "bytes_per_launch": w.append_bytes(with_q=True),
+            "avg_launch_ms": g["append_ms"],
+        },
+        "kernel_ms_per_layer": {"append": g["append_ms"], "attn": g["attn_ms"], "merge": g["merge_ms"]},
+    }
+    if not args.skip_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(args, w)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -125,6 +125,10 @@ int sdv2_kv_append_rope(const sdv2_append_params* p);
  * go through `workspace` (size from sdv2_swa_attn_workspace_bytes) and are
  * merged by a second kernel on the same stream.
  * ---------------------------------------------------------------------- */
+#define SDV2_STAGE_ALL 0
+#define SDV2_STAGE_PARTIAL 1
+#define SDV2_STAGE_MERGE 2
+
 typedef struct sdv2_attn_params {
   const void* q;               /* [B,S,H,128] bf16 (roped)                     */
   const void* k_cache;         /* [B,L,H,128] bf16 view of the cache           */
@@ -135,6 +139,9 @@ typedef struct sdv2_attn_params {
   int32_t rows, q_tokens, heads, head_dim;        /* B, S, H, 128              */
   int32_t max_seq_len;                            /* L = k_cache.shape[1]      */
   int32_t num_splits;          /* 0 = choose from the shape                    */
+  int32_t stages;              /* 0 = whole operator; SDV2_STAGE_PARTIAL /     */
+                               /* SDV2_STAGE_MERGE run one of the two kernels  */
+                               /* of a split call (for timing them apart)      */
   float softmax_scale;         /* <= 0 selects 1/sqrt(head_dim)                */
   void* workspace;             /* device scratch, 256-byte aligned             */
   size_t workspace_bytes;

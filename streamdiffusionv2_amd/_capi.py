@@ -22,6 +22,8 @@ SDV2_ERR_OUT_OF_RANGE = -3
 SDV2_ERR_WORKSPACE = -4
 SDV2_ERR_LAUNCH = -5
 
+STAGE_ALL, STAGE_PARTIAL, STAGE_MERGE = 0, 1, 2
+
 DTYPE_BF16 = 0
 DTYPE_F32 = 1
 
@@ -71,6 +73,7 @@ class AttnParams(C.Structure):
         ("rows", C.c_int32), ("q_tokens", C.c_int32), ("heads", C.c_int32), ("head_dim", C.c_int32),
         ("max_seq_len", C.c_int32),
         ("num_splits", C.c_int32),
+        ("stages", C.c_int32),
         ("softmax_scale", C.c_float),
         ("workspace", C.c_void_p),
         ("workspace_bytes", C.c_size_t),

@@ -60,11 +60,80 @@ def _host_ints(value, slot: str, rows: Optional[int] = None) -> List[int]:
     return out
 
 
-class CausalWanSelfAttention(nn.Module):
+class RingKVPath:
+    """The KV-cache path without the projections around it: ring state
+    (``sink_size``, ``adapt_sink_thr``, ``evict_idx``; causal_model.py:177-179)
+    plus :meth:`attend`.  ``CausalWanSelfAttention`` mixes it in; benchmarks and
+    tests that feed q/k/v directly use it on its own."""
+
+    def __init__(self, sink_size: int = 3, adapt_sink_thr: float = -1):
+        self.sink_size = sink_size
+        self.adapt_sink_thr = adapt_sink_thr
+        self.evict_idx: Optional[List[List[int]]] = None
+
+    def attend(self, q, k, v, grid_sizes, freqs, kv_cache, current_start,
+               return_roped_query: bool = False):
+        """RoPE + ring append + attention for q/k/v [B, S, H, 128]
+        (causal_model.py:250-384)."""
+        rows = q.shape[0]
+        grids = _host_ints(grid_sizes, "grid")
+        f, h, w = grids[0], grids[1], grids[2]
+        for r in range(1, len(grids) // 3):
+            if tuple(grids[3 * r:3 * r + 3]) != (f, h, w):
+                raise RuntimeError("all rows of a call must share one (F, H, W) grid")
+        frame_tokens = h * w
+        starts = _host_ints(current_start, "start", rows)
+        if len(starts) != rows:
+            raise RuntimeError(f"current_start has {len(starts)} entries for {rows} rows")
+
+        cache_rows = kv_cache["k"].shape[0]
+        if self.evict_idx is None:
+            self.evict_idx = [[]]
+        if len(self.evict_idx) < cache_rows:
+            self.evict_idx = [list(self.evict_idx[0]) for _ in range(cache_rows)]
+
+        if self.sink_size * frame_tokens > 0 and self.adapt_sink_thr > -1 and q.shape[1] <= frame_tokens:
+            raise NotImplementedError(
+                "adaptive sink refresh (causal_model.py:284-299) is not built yet; "
+                "set adapt_sink_thr = -1 for permanent sinks"
+            )
+
+        plan = ring.plan_append(kv_cache, self.evict_idx, starts, q.shape[1], frame_tokens, self.sink_size)
+        table = ops.device_freqs(freqs, q.device)
+        roped_q = ops.kv_append_rope(
+            q, k, v, kv_cache["k"], kv_cache["v"], table, (f, h, w),
+            [c // frame_tokens for c in starts], plan.dst_start,
+            global_end_index=kv_cache["global_end_index"],
+            local_end_index=kv_cache["local_end_index"],
+            new_global_end=plan.new_global_end,
+            new_local_end=plan.new_local_end,
+        )
+        span = plan.max_seq_len
+        seq = None
+        if any(n != span for n in plan.new_local_end):
+            # rows differ only while the stream batch is still filling; the
+            # lengths are a handful of host ints, shipped asynchronously
+            seq = torch.tensor(plan.new_local_end, dtype=torch.int32).to(q.device, non_blocking=True)
+        if roped_q.dtype == torch.bfloat16:
+            out = ops.swa_attention(roped_q, kv_cache["k"][:, :span], kv_cache["v"][:, :span], seq)
+        else:
+            # fp32 storage is a plumbing mode (the reference's CPU-runnable
+            # configuration): RoPE, cache and indices stay fp32 and bit-exact,
+            # the attention kernel computes in bf16 on down-cast copies.
+            out = ops.swa_attention(
+                roped_q.bfloat16(), kv_cache["k"][:, :span].bfloat16(), kv_cache["v"][:, :span].bfloat16(), seq
+            ).to(roped_q.dtype)
+        self.last_plan = plan
+        if return_roped_query:
+            return out, roped_q
+        return out
+
+
+class CausalWanSelfAttention(nn.Module, RingKVPath):
 
     def __init__(self, dim, num_heads, window_size=(-1, -1), qk_norm=True, eps=1e-6):
         assert dim % num_heads == 0
-        super().__init__()
+        nn.Module.__init__(self)
         self.dim = dim
         self.num_heads = num_heads
         self.head_dim = dim // num_heads
@@ -111,52 +180,3 @@ class CausalWanSelfAttention(nn.Module):
         v = self.v(x).view(b, s, n, d)
         out = self.attend(q, k, v, grid_sizes, freqs, kv_cache, current_start)
         return self.o(out.flatten(2))
-
-    # ------------------------------------------------------------------
-    def attend(self, q, k, v, grid_sizes, freqs, kv_cache, current_start,
-               return_roped_query: bool = False):
-        """The path proper, after the projections: RoPE + ring append +
-        attention for q/k/v [B, S, H, 128] (causal_model.py:250-384)."""
-        rows = q.shape[0]
-        grids = _host_ints(grid_sizes, "grid")
-        f, h, w = grids[0], grids[1], grids[2]
-        for r in range(1, len(grids) // 3):
-            if tuple(grids[3 * r:3 * r + 3]) != (f, h, w):
-                raise RuntimeError("all rows of a call must share one (F, H, W) grid")
-        frame_tokens = h * w
-        starts = _host_ints(current_start, "start", rows)
-        if len(starts) != rows:
-            raise RuntimeError(f"current_start has {len(starts)} entries for {rows} rows")
-
-        cache_rows = kv_cache["k"].shape[0]
-        if self.evict_idx is None:
-            self.evict_idx = [[]]
-        if len(self.evict_idx) < cache_rows:
-            self.evict_idx = [list(self.evict_idx[0]) for _ in range(cache_rows)]
-
-        if self.sink_size * frame_tokens > 0 and self.adapt_sink_thr > -1 and q.shape[1] <= frame_tokens:
-            raise NotImplementedError(
-                "adaptive sink refresh (causal_model.py:284-299) is not built yet; "
-                "set adapt_sink_thr = -1 for permanent sinks"
-            )
-
-        plan = ring.plan_append(kv_cache, self.evict_idx, starts, q.shape[1], frame_tokens, self.sink_size)
-        table = ops.device_freqs(freqs, q.device)
-        roped_q = ops.kv_append_rope(
-            q, k, v, kv_cache["k"], kv_cache["v"], table, (f, h, w),
-            [c // frame_tokens for c in starts], plan.dst_start,
-            global_end_index=kv_cache["global_end_index"],
-            local_end_index=kv_cache["local_end_index"],
-            new_global_end=plan.new_global_end,
-            new_local_end=plan.new_local_end,
-        )
-        span = plan.max_seq_len
-        seq = None
-        if any(n != span for n in plan.new_local_end):
-            # rows differ only while the stream batch is still filling; the
-            # lengths are a handful of host ints, shipped asynchronously
-            seq = torch.tensor(plan.new_local_end, dtype=torch.int32).to(q.device, non_blocking=True)
-        out = ops.swa_attention(roped_q, kv_cache["k"][:, :span], kv_cache["v"][:, :span], seq)
-        if return_roped_query:
-            return out, roped_q
-        return out

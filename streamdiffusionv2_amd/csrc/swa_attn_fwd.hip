@@ -402,6 +402,8 @@ extern "C" int sdv2_swa_attn_fwd(const sdv2_attn_params* p) {
   int splits = p->num_splits > 0 ? p->num_splits
                                  : sdv2_swa_attn_default_splits(p->rows, p->q_tokens, p->heads, p->max_seq_len);
   if (splits > 64) return SDV2_ERR_INVALID_ARG;
+  if (p->stages < SDV2_STAGE_ALL || p->stages > SDV2_STAGE_MERGE) return SDV2_ERR_INVALID_ARG;
+  if (p->stages != SDV2_STAGE_ALL && splits == 1) return SDV2_ERR_INVALID_ARG;
   if ((int64_t)p->rows * splits > 65535) return SDV2_ERR_INVALID_ARG;
 
   AttnKernelArgs a{};
@@ -428,9 +430,11 @@ extern "C" int sdv2_swa_attn_fwd(const sdv2_attn_params* p) {
 
   hipStream_t stream = static_cast<hipStream_t>(p->stream);
   dim3 grid((p->q_tokens + kQTile - 1) / kQTile, p->heads, p->rows * splits);
-  hipLaunchKernelGGL(swa_attn_fwd_kernel, grid, dim3(kThreads), 0, stream, a);
-  if (hipGetLastError() != hipSuccess) return SDV2_ERR_LAUNCH;
-  if (splits > 1) {
+  if (p->stages != SDV2_STAGE_MERGE) {
+    hipLaunchKernelGGL(swa_attn_fwd_kernel, grid, dim3(kThreads), 0, stream, a);
+    if (hipGetLastError() != hipSuccess) return SDV2_ERR_LAUNCH;
+  }
+  if (splits > 1 && p->stages != SDV2_STAGE_PARTIAL) {
     const int64_t nq = (int64_t)p->rows * p->heads * p->q_tokens;
     hipLaunchKernelGGL(swa_attn_merge_kernel, dim3((unsigned)((nq + 15) / 16)), dim3(256), 0, stream, a);
     if (hipGetLastError() != hipSuccess) return SDV2_ERR_LAUNCH;

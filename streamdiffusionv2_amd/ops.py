@@ -176,6 +176,7 @@ def swa_attention(
     num_splits: int = 0,
     softmax_scale: Optional[float] = None,
     workspace: Optional[torch.Tensor] = None,
+    stages: int = _capi.STAGE_ALL,
 ) -> torch.Tensor:
     """out[b] = softmax(q[b] k_cache[b,:seq_lens[b]]^T * scale) v_cache[b,:seq_lens[b]].
 
@@ -212,6 +213,7 @@ def swa_attention(
     p.rows, p.q_tokens, p.heads, p.head_dim = rows, q_tokens, heads, HEAD_DIM
     p.max_seq_len = max_seq_len
     p.num_splits = num_splits
+    p.stages = stages
     p.softmax_scale = float(softmax_scale) if softmax_scale else 0.0
     if need:
         p.workspace = workspace.data_ptr()

@@ -1,0 +1,114 @@
+"""The C-ABI library loads without a GPU, exports every function that
+include/sdv2kv.h declares, and rejects bad arguments before touching HIP."""
+import ctypes as C
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+from streamdiffusionv2_amd import _capi
+
+HEADER = os.path.join(os.path.dirname(os.path.dirname(__file__)), "include", "sdv2kv.h")
+
+
+def declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sdv2_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_functions_are_exported():
+    names = declared_functions()
+    assert sorted(_capi.EXPORTED_SYMBOLS) == names
+    lib = _capi.lib()
+    for n in names:
+        assert hasattr(lib, n), n
+    assert lib.sdv2_abi_version() == _capi.ABI_VERSION
+
+
+def test_header_constants_match_binding():
+    text = open(HEADER).read()
+    assert int(re.search(r"#define SDV2_MAX_ROWS (\d+)", text).group(1)) == _capi.MAX_ROWS
+    assert int(re.search(r"#define SDV2_HEAD_DIM (\d+)", text).group(1)) == _capi.HEAD_DIM
+    for name in ("INVALID_ARG", "UNSUPPORTED", "OUT_OF_RANGE", "WORKSPACE", "LAUNCH"):
+        val = int(re.search(rf"SDV2_ERR_{name} = (-\d+)", text).group(1))
+        assert getattr(_capi, f"SDV2_ERR_{name}") == val
+    # struct field order of the binding follows the header
+    for struct, cls in (("sdv2_append_params", _capi.AppendParams), ("sdv2_attn_params", _capi.AttnParams)):
+        body = re.search(rf"typedef struct {struct} \{{(.*?)\}} {struct};", text, flags=re.S).group(1)
+        body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+        fields = []
+        for decl in body.split(";"):
+            decl = decl.strip()
+            if not decl:
+                continue
+            names = re.sub(r"^(const\s+)?[A-Za-z0-9_]+\s*\**", "", decl)
+            fields += [n.strip().lstrip("*") for n in names.split(",")]
+        assert fields == [f[0] for f in cls._fields_], struct
+
+
+def test_argument_validation_without_gpu():
+    lib = _capi.lib()
+    assert lib.sdv2_kv_append_rope(None) == _capi.SDV2_ERR_INVALID_ARG
+    assert lib.sdv2_swa_attn_fwd(None) == _capi.SDV2_ERR_INVALID_ARG
+    p = _capi.AppendParams()
+    p.head_dim = 64
+    assert lib.sdv2_kv_append_rope(C.byref(p)) == _capi.SDV2_ERR_UNSUPPORTED
+    p.head_dim, p.dtype = 128, 7
+    assert lib.sdv2_kv_append_rope(C.byref(p)) == _capi.SDV2_ERR_UNSUPPORTED
+    p.dtype, p.rows, p.tokens, p.heads = 0, _capi.MAX_ROWS + 1, 8, 1
+    assert lib.sdv2_kv_append_rope(C.byref(p)) == _capi.SDV2_ERR_INVALID_ARG
+    p.rows, p.grid_f, p.grid_h, p.grid_w = 1, 1, 2, 3      # 6 != 8 tokens
+    assert lib.sdv2_kv_append_rope(C.byref(p)) == _capi.SDV2_ERR_INVALID_ARG
+    a = _capi.AttnParams()
+    a.head_dim = 96
+    assert lib.sdv2_swa_attn_fwd(C.byref(a)) == _capi.SDV2_ERR_UNSUPPORTED
+    a.head_dim, a.rows, a.q_tokens, a.heads, a.max_seq_len = 128, 1, 4, 1, 8
+    assert lib.sdv2_swa_attn_fwd(C.byref(a)) == _capi.SDV2_ERR_INVALID_ARG     # null tensors
+    assert b"workspace" in lib.sdv2_status_string(_capi.SDV2_ERR_WORKSPACE)
+    with pytest.raises(RuntimeError, match="status -3"):
+        _capi.check(_capi.SDV2_ERR_OUT_OF_RANGE, "x")
+
+
+def test_split_heuristic_and_workspace_size():
+    lib = _capi.lib()
+    assert lib.sdv2_swa_attn_workspace_bytes(1, 1560, 12, 9360, 1) == 0
+    s = lib.sdv2_swa_attn_default_splits(1, 1560, 12, 9360)
+    assert s >= 2
+    nq = 1560 * 12
+    need = lib.sdv2_swa_attn_workspace_bytes(1, 1560, 12, 9360, s)
+    assert need >= s * nq * (128 + 1) * 4
+    assert lib.sdv2_swa_attn_default_splits(4, 4680, 12, 18720) == 1       # enough query tiles already
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    monkeypatch.setattr(_capi, "_LIB", None)
+    monkeypatch.setattr(_capi, "LIB_PATH", tmp_path / "nope.so")
+    with pytest.raises(ImportError, match="no fallback"):
+        _capi.lib()
+
+
+def test_cpu_tensors_are_refused():
+    from streamdiffusionv2_amd import ops
+
+    q = torch.zeros(1, 8, 1, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ops.swa_attention(q, q, q)
+
+
+def test_module_signature_matches_reference():
+    from streamdiffusionv2_amd.attention import CausalWanSelfAttention
+
+    # models/wan/causal_model.py:162-167 and :189-200
+    assert list(inspect.signature(CausalWanSelfAttention.__init__).parameters) == [
+        "self", "dim", "num_heads", "window_size", "qk_norm", "eps"]
+    assert list(inspect.signature(CausalWanSelfAttention.forward).parameters) == [
+        "self", "x", "seq_lens", "grid_sizes", "freqs", "block_mask", "kv_cache",
+        "current_start", "current_end", "causal_rope_cache"]
+    m = CausalWanSelfAttention(256, 2)
+    assert (m.sink_size, m.adapt_sink_thr, m.evict_idx) == (3, -1, None)
+    assert {n for n, _ in m.named_children()} == {"q", "k", "v", "o", "norm_q", "norm_k"}
+    with pytest.raises(NotImplementedError):
+        m(torch.zeros(1, 4, 256), None, None, None, None, kv_cache=None)
