@@ -29,6 +29,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <utility>
+
 #include "sdv2kv.h"
 #include "sdv2kv_internal.h"
 
@@ -41,6 +43,7 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 typedef __attribute__((address_space(3))) char lds_char;
 
 constexpr int kD = SDV2_HEAD_DIM;           // 128
@@ -84,37 +87,204 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
 }
 
-struct TileRegs {
-  u32x4 k[4];
-  u32x4 v[4];
+// ---------------------------------------------------------------------------
+// Tile loader: global -> LDS without passing through registers
+// (global_load_lds_dwordx4).  One wave-wide instruction deposits 64 x 16 bytes
+// at consecutive LDS addresses, i.e. four 256-byte key rows.  Instruction i
+// (0..15, four per wave) fills rows 4i..4i+3; lane l lands on row 4i + l/16,
+// physical chunk l%16, so it must fetch logical chunk (l%16) ^ g(row).
+// ---------------------------------------------------------------------------
+// ---------------------------------------------------------------------------
+// LDS reads with hand-placed waits.  The compiler treats every LDS access as
+// possibly aliasing an in-flight global->LDS transfer and would drain all
+// counters before each dependent MFMA; issuing the reads as asm and tying an
+// explicit s_waitcnt to the fragment about to be consumed keeps several reads
+// in flight behind the matrix pipe.  LDS returns data in issue order, so
+// lgkmcnt(N) means "all but the newest N reads have landed".
+// ---------------------------------------------------------------------------
+template <int... I, typename F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(std::make_integer_sequence<int, N>{}, f);
+}
+
+template <int kOffset>
+__device__ __forceinline__ u32x4 lds_read_b128(uint32_t addr) {
+  u32x4 r;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(kOffset));
+  return r;
+}
+template <int kOffset>
+__device__ __forceinline__ u32x2 lds_read_tr16_b64(uint32_t addr) {
+  u32x2 r;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(kOffset));
+  return r;
+}
+template <int kPending>
+__device__ __forceinline__ void wait_lds(u32x4& frag) {
+  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(frag) : "n"(kPending));
+}
+
+struct LoaderOffsets {
+  uint32_t k[4];   // byte offsets from the tile's first key row, per instruction
+  uint32_t v[4];
 };
 
-// Each thread moves four 16-byte chunks of K and of V per tile: rows
-// tid/16 + 16 i, chunk tid % 16.  Rows past the valid length are clamped to
-// the last valid key (their scores are masked later), so nothing is read
-// outside the rows the caller declared valid.
-__device__ __forceinline__ void load_tile(TileRegs& t, const uint16_t* kbase, const uint16_t* vbase,
-                                          int64_t k_tok_stride, int64_t v_tok_stride,
-                                          int key0, int last_key, int tid) {
-  const int c = tid & 15;
+__device__ __forceinline__ void dma16(const char* g, lds_char* l) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
+                                   (__attribute__((address_space(3))) void*)l, 16, 0, 0);
+}
+
+// full tile: every row is valid, addresses are tile base + precomputed offsets
+__device__ __forceinline__ void load_tile_dma(const LoaderOffsets& o, const char* ktile, const char* vtile,
+                                              lds_char* stage, int wave_u) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    int key = key0 + (tid >> 4) + 16 * i;
-    key = key < last_key ? key : last_key;
-    t.k[i] = *reinterpret_cast<const u32x4*>(kbase + key * k_tok_stride + c * 8);
-    t.v[i] = *reinterpret_cast<const u32x4*>(vbase + key * v_tok_stride + c * 8);
+  for (int j = 0; j < 4; ++j) {
+    dma16(ktile + o.k[j], stage + (wave_u * 4 + j) * 1024);
+    dma16(vtile + o.v[j], stage + kTileBytes + (wave_u * 4 + j) * 1024);
   }
 }
 
-__device__ __forceinline__ void store_tile(const TileRegs& t, lds_char* stage, int tid) {
-  const int c = tid & 15;
+// last, partial tile: rows at or past the valid length are redirected to the
+// last valid key (their scores are masked), so nothing outside the rows the
+// caller declared valid is read.
+__device__ __forceinline__ void load_tile_dma_tail(const char* kbase, const char* vbase, int64_t k_tok_bytes,
+                                                   int64_t v_tok_bytes, int key0, int last_key,
+                                                   lds_char* stage, int wave_u, int lane) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = (tid >> 4) + 16 * i;
-    const int off = r * 256 + ((c ^ swz(r)) << 4);
-    *reinterpret_cast<__attribute__((address_space(3))) u32x4*>(stage + off) = t.k[i];
-    *reinterpret_cast<__attribute__((address_space(3))) u32x4*>(stage + kTileBytes + off) = t.v[i];
+  for (int j = 0; j < 4; ++j) {
+    const int r = 4 * (wave_u * 4 + j) + (lane >> 4);
+    int key = key0 + r;
+    key = key < last_key ? key : last_key;
+    const int chunk = (lane & 15) ^ swz(r);
+    dma16(kbase + key * k_tok_bytes + chunk * 16, stage + (wave_u * 4 + j) * 1024);
+    dma16(vbase + key * v_tok_bytes + chunk * 16, stage + kTileBytes + (wave_u * 4 + j) * 1024);
   }
+}
+
+__device__ __forceinline__ void wait_vmem_and_sync() {
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's DMA has landed
+  __syncthreads();
+}
+
+struct SoftmaxState {
+  float m;   // running max of the raw scores of this lane's query
+  float l;   // this lane's share of the running sum
+};
+
+// One 64-key tile from LDS stage `kBuf` (compile-time, so every LDS address is
+// register + immediate).
+template <int kBuf>
+__device__ __forceinline__ void process_tile(const uint32_t (&k_addr)[8], const uint32_t (&v_addr)[4][2],
+                                             const bf16x8 (&qf)[8], f32x16 (&oacc)[4], SoftmaxState& st,
+                                             float c2, int key0, int seq, int hf) {
+  constexpr int kBase = kBuf * kStageBytes;
+  constexpr int vBase = kBuf * kStageBytes + kTileBytes;
+
+  // ---- S^T = K Q^T : two 32-key blocks --------------------------------
+  // 16 MFMAs, the two accumulators alternating; K fragments are fetched from
+  // LDS kAhead MFMAs ahead.  Step s covers d-step s/2 of key block s%2.
+  f32x16 sacc[2];
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.f;
+  constexpr int kAhead = 4;
+  u32x4 kf[16];
+  static_for<kAhead>([&](auto ic) {
+    constexpr int s = decltype(ic)::value;
+    kf[s] = lds_read_b128<kBase + (s & 1) * 32 * 256>(k_addr[s >> 1]);
+  });
+  static_for<16>([&](auto ic) {
+    constexpr int s = decltype(ic)::value;
+    if constexpr (s + kAhead < 16)
+      kf[s + kAhead] = lds_read_b128<kBase + ((s + kAhead) & 1) * 32 * 256>(k_addr[(s + kAhead) >> 1]);
+    wait_lds<(s + kAhead < 16) ? kAhead : 15 - s>(kf[s]);
+    sacc[s & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[s]), qf[s >> 1],
+                                                          sacc[s & 1], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  });
+
+  // first V^T fragments: issued now, they land while the softmax runs.
+  // Step s covers key step s/4 (16 keys) and d block s%4.
+  constexpr int vAhead = 4;
+  u32x4 vf[16];
+  auto v_frag = [&](auto ic) {
+    constexpr int s = decltype(ic)::value;
+    constexpr int kk = s >> 2, db = s & 3;
+    const u32x2 lo = lds_read_tr16_b64<vBase + kk * 16 * 256>(v_addr[db][0]);
+    const u32x2 hi = lds_read_tr16_b64<vBase + kk * 16 * 256>(v_addr[db][1]);
+    vf[s] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3);
+  };
+  static_for<vAhead>(v_frag);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- mask the tail of the last tile ---------------------------------
+  if (key0 + kKTile > seq) {
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int key = key0 + kb * 32 + 8 * (i >> 2) + 4 * hf + (i & 3);
+        if (key >= seq) sacc[kb][i] = -INFINITY;
+      }
+  }
+
+  // ---- online softmax, one query per lane ------------------------------
+  float mloc = sacc[0][0];
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, sacc[kb][i]);
+  mloc = half_max(mloc);
+  const float m_new = fmaxf(st.m, mloc);
+  const float alpha = __builtin_amdgcn_exp2f((st.m - m_new) * c2);
+  const float mc = m_new * c2;
+  st.m = m_new;
+  float psum = 0.f;
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][i], c2, -mc));
+      sacc[kb][i] = p;
+      psum += p;
+    }
+  st.l = st.l * alpha + psum;
+  if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
+  }
+
+  // ---- P^T as the B operand: accumulator registers 8*step..8*step+7 ----
+  bf16x8 pf[2][2];
+#pragma unroll
+  for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+    for (int s2 = 0; s2 < 2; ++s2) {
+      union { uint32_t u[4]; bf16x8 v; } pk;
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        pk.u[j] = pack_bf16x2(sacc[kb][8 * s2 + 2 * j], sacc[kb][8 * s2 + 2 * j + 1]);
+      pf[kb][s2] = pk.v;
+    }
+
+  // ---- O^T += V^T P^T ----------------------------------------------------
+  __builtin_amdgcn_sched_barrier(0);
+  static_for<16>([&](auto ic) {
+    constexpr int s = decltype(ic)::value;
+    if constexpr (s + vAhead < 16) v_frag(std::integral_constant<int, s + vAhead>{});
+    wait_lds<(s + vAhead < 16) ? 2 * vAhead : 2 * (15 - s)>(vf[s]);
+    constexpr int kk = s >> 2, db = s & 3;
+    oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf[s]), pf[kk >> 1][kk & 1],
+                                                       oacc[db], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+  });
 }
 
 __global__ __launch_bounds__(kThreads, 2)
@@ -125,6 +295,7 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int hf = lane >> 5;                 // which half of the wave
   const int qtile = blockIdx.x;
   const int head = blockIdx.y;
@@ -140,6 +311,31 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   int tile_end = tile_begin + per_split;
   tile_end = tile_end < ntiles ? tile_end : ntiles;
 
+  const char* kbase = reinterpret_cast<const char*>(a.k + row * a.k_st.row + head * a.k_st.head);
+  const char* vbase = reinterpret_cast<const char*>(a.v + row * a.v_st.row + head * a.v_st.head);
+  const int64_t k_tok_bytes = a.k_st.token * 2;
+  const int64_t v_tok_bytes = a.v_st.token * 2;
+
+  LoaderOffsets lo;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int r = 4 * (wave * 4 + j) + (lane >> 4);
+    const int chunk = (lane & 15) ^ swz(r);
+    lo.k[j] = (uint32_t)(r * k_tok_bytes + chunk * 16);
+    lo.v[j] = (uint32_t)(r * v_tok_bytes + chunk * 16);
+  }
+
+  auto issue_tile = [&](int t, int buf) {
+    const int key0 = t * kKTile;
+    lds_char* stage = lds + buf * kStageBytes;
+    if (key0 + kKTile <= seq)
+      load_tile_dma(lo, kbase + key0 * k_tok_bytes, vbase + key0 * v_tok_bytes, stage, wave_u);
+    else
+      load_tile_dma_tail(kbase, vbase, k_tok_bytes, v_tok_bytes, key0, seq - 1, stage, wave_u, lane);
+  };
+
+  if (tile_begin < tile_end) issue_tile(tile_begin, 0);
+
   // ---- this lane's query row, as the B operand of S^T = K Q^T -------------
   const int q_row = qtile * kQTile + wave * kQRowsPerWave + (lane & 31);
   const int q_row_c = q_row < a.q_tokens ? q_row : a.q_tokens - 1;
@@ -148,22 +344,20 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
 #pragma unroll
   for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
 
-  const uint16_t* kbase = a.k + row * a.k_st.row + head * a.k_st.head;
-  const uint16_t* vbase = a.v + row * a.v_st.row + head * a.v_st.head;
-
   // ---- per-lane LDS read offsets -------------------------------------------
   // K (A operand): key = kb*32 + lane%32, chunk = 2*ks + hf
-  int k_off[8];
+  const uint32_t lds_addr0 = (uint32_t)(uintptr_t)lds;
+  uint32_t k_addr[8];
   {
     const int r = lane & 31;
     const int base = r * 256 + ((hf ^ swz(r)) << 4);
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) k_off[ks] = base ^ (ks << 5);
+    for (int ks = 0; ks < 8; ++ks) k_addr[ks] = lds_addr0 + (uint32_t)(base ^ (ks << 5));
   }
   // V^T (A operand) through the transposing read: in each group of 16 lanes,
   // lane i supplies the address of key (i / 4), 8 bytes at d-offset 4 * (i % 4);
   // it receives d = i, keys 0..3.  Group = (hf, dhalf).
-  int v_off[4][2];
+  uint32_t v_addr[4][2];
   {
     const int i16 = lane & 15;
     const int dhalf = (lane >> 4) & 1;
@@ -174,7 +368,7 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
       for (int j = 0; j < 2; ++j) {
         const int r = 8 * j + 4 * hf + krow;                 // + 16 * kk added as an immediate
         const int c = db * 4 + dhalf * 2 + ((i16 & 3) >> 1);
-        v_off[db][j] = kTileBytes + r * 256 + ((c ^ swz(r)) << 4) + (i16 & 1) * 8;
+        v_addr[db][j] = lds_addr0 + (uint32_t)(r * 256 + ((c ^ swz(r)) << 4) + (i16 & 1) * 8);
       }
   }
 
@@ -183,110 +377,24 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   for (int db = 0; db < 4; ++db)
 #pragma unroll
     for (int i = 0; i < 16; ++i) oacc[db][i] = 0.f;
-  float m_run = -INFINITY;    // running max of raw scores (this lane's query)
-  float l_run = 0.f;          // this lane's share of the running sum
-
+  SoftmaxState st{-INFINITY, 0.f};
   const float c2 = a.scale_log2;
 
-  if (tile_begin < tile_end) {
-    TileRegs stage_regs;
-    load_tile(stage_regs, kbase, vbase, a.k_st.token, a.v_st.token, tile_begin * kKTile, seq - 1, tid);
-    store_tile(stage_regs, lds, tid);
-    __syncthreads();
+  wait_vmem_and_sync();   // first tile and the Q fragments have arrived
 
-    for (int t = tile_begin; t < tile_end; ++t) {
-      const int buf = (t - tile_begin) & 1;
-      lds_char* cur = lds + buf * kStageBytes;
-      const bool has_next = t + 1 < tile_end;
-      if (has_next)
-        load_tile(stage_regs, kbase, vbase, a.k_st.token, a.v_st.token, (t + 1) * kKTile, seq - 1, tid);
-
-      // ---- S^T = K Q^T : two 32-key blocks --------------------------------
-      f32x16 sacc[2];
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks) {
-          const bf16x8 kf = *reinterpret_cast<__attribute__((address_space(3))) const bf16x8*>(
-              cur + k_off[ks] + kb * 32 * 256);
-          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc[kb], 0, 0, 0);
-        }
-      }
-
-      // ---- mask the tail of the last tile ---------------------------------
-      const int key0 = t * kKTile;
-      if (key0 + kKTile > seq) {
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) {
-            const int key = key0 + kb * 32 + 8 * (i >> 2) + 4 * hf + (i & 3);
-            if (key >= seq) sacc[kb][i] = -INFINITY;
-          }
-      }
-
-      // ---- online softmax, one query per lane ------------------------------
-      float mloc = sacc[0][0];
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, sacc[kb][i]);
-      mloc = half_max(mloc);
-      const float m_new = fmaxf(m_run, mloc);
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c2);
-      const float mc = m_new * c2;
-      m_run = m_new;
-      float psum = 0.f;
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-          const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][i], c2, -mc));
-          sacc[kb][i] = p;
-          psum += p;
-        }
-      l_run = l_run * alpha + psum;
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-        for (int db = 0; db < 4; ++db)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
-      }
-
-      // ---- P^T as the B operand: accumulator registers 8*step..8*step+7 ----
-      bf16x8 pf[2][2];
-#pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-        for (int st = 0; st < 2; ++st) {
-          union { uint32_t u[4]; bf16x8 v; } pk;
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-            pk.u[j] = pack_bf16x2(sacc[kb][8 * st + 2 * j], sacc[kb][8 * st + 2 * j + 1]);
-          pf[kb][st] = pk.v;
-        }
-
-      // ---- O^T += V^T P^T ----------------------------------------------------
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-#pragma unroll
-        for (int db = 0; db < 4; ++db) {
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (__attribute__((address_space(3))) s16x4*)(cur + v_off[db][0] + kk * 16 * 256));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-              (__attribute__((address_space(3))) s16x4*)(cur + v_off[db][1] + kk * 16 * 256));
-          const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              __builtin_bit_cast(bf16x8, both), pf[kk >> 1][kk & 1], oacc[db], 0, 0, 0);
-        }
-      }
-
-      if (has_next) store_tile(stage_regs, lds + (buf ^ 1) * kStageBytes, tid);
-      __syncthreads();
-    }
+  // Two tiles per trip so the LDS stage is a compile-time constant.
+  for (int t = tile_begin; t < tile_end; t += 2) {
+    if (t + 1 < tile_end) issue_tile(t + 1, 1);
+    process_tile<0>(k_addr, v_addr, qf, oacc, st, c2, t * kKTile, seq, hf);
+    wait_vmem_and_sync();
+    if (t + 1 >= tile_end) break;
+    if (t + 2 < tile_end) issue_tile(t + 2, 0);
+    process_tile<1>(k_addr, v_addr, qf, oacc, st, c2, (t + 1) * kKTile, seq, hf);
+    wait_vmem_and_sync();
   }
+
+  float m_run = st.m;
+  float l_run = st.l;
 
   // ---- epilogue ---------------------------------------------------------------
   const float l_tot = half_sum(l_run);
