@@ -8,19 +8,28 @@
 // has to be unrolled.
 //
 // Work decomposition
-//   workgroup = 4 waves, 128 query rows of one (row, head); wave w owns rows
-//   32w..32w+31.  Keys stream through LDS in tiles of 64 (K 16 KB + V 16 KB,
-//   double buffered, 64 KB per workgroup, two workgroups per CU).
+//   workgroup = 4 waves = 256 query rows of one (row, head), one workgroup per
+//   CU; wave w owns rows 64w..64w+63 as two 32-row blocks, so every K / V
+//   fragment fetched from LDS feeds two MFMAs.  Keys stream through LDS in
+//   tiles of 64 (K 16 KB + V 16 KB), three buffers each, filled two tiles
+//   ahead by global->LDS transfers that never touch registers.
 //
 // Matrix layout (v_mfma_f32_32x32x16_bf16, D = A(32x16) * B(16x32) + C):
-//   S^T = K Q^T   A = K tile rows (16 B per lane straight from LDS),
-//                 B = Q, held in registers for the whole kernel.
+//   S^T = K Q^T   A = K tile rows (ds_read_b128), B = Q, in registers for the
+//                 whole kernel.
 //   O^T = V^T P^T A = V^T read with ds_read_b64_tr_b16 (LDS transpose load),
 //                 B = P^T, which is exactly the S^T accumulator layout after
 //                 packing to bf16 — no cross-lane movement between the GEMMs.
-//   In both products a lane owns ONE query (column lane%32), so the online
-//   softmax statistics are per-lane scalars; the only cross-lane step is one
-//   exchange between lane halves (v_permlane32_swap).
+//   In both products a lane owns ONE query per block (column lane%32), so the
+//   softmax statistics are per-lane scalars.
+//
+// Softmax.  exp2 of the scaled scores is taken without subtracting a running
+// maximum: the weights stay in fp32 / bf16 range as long as the scaled scores
+// stay within about +-100 in log2 units, which every sane attention input
+// does, and the result is mathematically the same.  Each wave checks its row
+// sums every slot; if any leaves [2^-100, 2^100] (or is NaN) the workgroup
+// finishes the fast pass, throws its result away and recomputes with the
+// conventional running-maximum recurrence (slow, exact for any finite input).
 //
 // LDS tile layout: row r (key) holds sixteen 16-byte chunks; chunk c is stored
 // at position c ^ g(r), g(r) = ((r & 3) << 2) | ((r >> 2) & 3).  That makes the
@@ -37,11 +46,11 @@
 namespace {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 typedef __attribute__((address_space(3))) char lds_char;
@@ -49,12 +58,24 @@ typedef __attribute__((address_space(3))) char lds_char;
 constexpr int kD = SDV2_HEAD_DIM;           // 128
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * 64;
-constexpr int kQRowsPerWave = 32;
-constexpr int kQTile = kWaves * kQRowsPerWave;   // 128
+constexpr int kQB = 2;                      // 32-row query blocks per wave
+constexpr int kQRowsPerWave = 32 * kQB;
+constexpr int kQTile = kWaves * kQRowsPerWave;   // 256
 constexpr int kKTile = 64;
 constexpr int kTileBytes = kKTile * kD * 2;      // 16 KB per matrix
-constexpr int kStageBytes = 2 * kTileBytes;      // K + V
+constexpr int kStages = 3;
+constexpr int kLdsBytes = 2 * kStages * kTileBytes;   // 96 KB
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kCuSlots = 256;               // one workgroup per CU
+
+// LDS map: kStages K tile buffers, then kStages V tile buffers.  The DS
+// instructions carry a 16-bit offset, so V fragment addresses are kept
+// relative to the first V buffer (kLdsVRel) with the base folded into the
+// per-lane address register.
+constexpr int kLdsK(int buf) { return buf * kTileBytes; }
+constexpr int kLdsVBase = kStages * kTileBytes;
+constexpr int kLdsVRel(int buf) { return buf * kTileBytes; }
+constexpr int kLdsV(int buf) { return kLdsVBase + kLdsVRel(buf); }
 
 struct AttnKernelArgs {
   const uint16_t* q;
@@ -71,10 +92,17 @@ struct AttnKernelArgs {
 
 __device__ __forceinline__ int swz(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
 
-// max over the two lanes that share a query column (lane and lane ^ 32)
+// v_max without the NaN-quieting canonicalisation fmaxf() drags in.
+__device__ __forceinline__ float vmax(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
+// exchange between the two lanes that share a query column (lane and lane ^ 32)
 __device__ __forceinline__ float half_max(float x) {
   auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  return vmax(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 __device__ __forceinline__ float half_sum(float x) {
   auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
@@ -87,13 +115,12 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
 }
 
-// ---------------------------------------------------------------------------
-// Tile loader: global -> LDS without passing through registers
-// (global_load_lds_dwordx4).  One wave-wide instruction deposits 64 x 16 bytes
-// at consecutive LDS addresses, i.e. four 256-byte key rows.  Instruction i
-// (0..15, four per wave) fills rows 4i..4i+3; lane l lands on row 4i + l/16,
-// physical chunk l%16, so it must fetch logical chunk (l%16) ^ g(row).
-// ---------------------------------------------------------------------------
+// acc + lo + hi of a packed bf16 pair (v_dot2c_f32_bf16 against (1, 1))
+__device__ __forceinline__ float add_bf16_pair(uint32_t packed, float acc) {
+  const bf16x2 ones = {(__bf16)1.0f, (__bf16)1.0f};
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, packed), ones, acc, false);
+}
+
 // ---------------------------------------------------------------------------
 // LDS reads with hand-placed waits.  The compiler treats every LDS access as
 // possibly aliasing an in-flight global->LDS transfer and would drain all
@@ -123,173 +150,323 @@ __device__ __forceinline__ u32x2 lds_read_tr16_b64(uint32_t addr) {
   asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(kOffset));
   return r;
 }
+// Optimisation passes may sink pure arithmetic down to its first use, which
+// here is a whole pipeline slot later.  Passing a value through an empty
+// volatile asm fixes the point by which it has to be computed.
+__device__ __forceinline__ void pin(float& x) { asm volatile("" : "+v"(x)); }
+__device__ __forceinline__ void pin(uint32_t& x) { asm volatile("" : "+v"(x)); }
+
+// The MFMAs of the fast pass are asm as well.  With one wave per SIMD the
+// compiler keeps every MFMA accumulator in the accumulation registers, but the
+// scores feed the vector ALU (which cannot read those) while the output tile
+// never does until the epilogue; naming the register class per product puts S
+// in VGPRs and O in AGPRs.  `kPending` is the s_waitcnt that makes the A
+// fragment valid (reads issued after it that may still be in flight); -1 = the
+// fragment was already waited for.  Nothing here is covered by the compiler's
+// hazard tracking: S is read by the vector ALU a full slot after its last
+// MFMA, P is written a full slot before the MFMA that reads it, and O is only
+// read after the final barrier, all far beyond the required wait states.
 template <int kPending>
-__device__ __forceinline__ void wait_lds(u32x4& frag) {
-  asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(frag) : "n"(kPending));
+__device__ __forceinline__ void mfma_s_first(f32x16& d, const u32x4& a, const bf16x8& b) {
+  if constexpr (kPending >= 0)
+    asm volatile("s_waitcnt lgkmcnt(%3)\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0"
+                 : "=&v"(d) : "v"(a), "v"(b), "n"(kPending));
+  else
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
+}
+template <int kPending>
+__device__ __forceinline__ void mfma_s(f32x16& d, const u32x4& a, const bf16x8& b) {
+  if constexpr (kPending >= 0)
+    asm volatile("s_waitcnt lgkmcnt(%3)\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0"
+                 : "+v"(d) : "v"(a), "v"(b), "n"(kPending));
+  else
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
+}
+template <int kPending>
+__device__ __forceinline__ void mfma_o(f32x16& d, const u32x4& a, const u32x4& b) {
+  if constexpr (kPending >= 0)
+    asm volatile("s_waitcnt lgkmcnt(%3)\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0"
+                 : "+a"(d) : "v"(a), "v"(b), "n"(kPending));
+  else
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(d) : "v"(a), "v"(b));
 }
 
-struct LoaderOffsets {
-  uint32_t k[4];   // byte offsets from the tile's first key row, per instruction
-  uint32_t v[4];
-};
-
-__device__ __forceinline__ void dma16(const char* g, lds_char* l) {
-  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g,
-                                   (__attribute__((address_space(3))) void*)l, 16, 0, 0);
+// ---------------------------------------------------------------------------
+// Tile loader: global -> LDS without passing through registers
+// (global_load_lds_dwordx4).  One wave-wide instruction deposits 64 x 16 bytes
+// at consecutive LDS addresses, i.e. four 256-byte key rows.  Instruction i
+// (0..15, four per wave) fills rows 4i..4i+3; lane l lands on row 4i + l/16,
+// physical chunk l%16, so it must fetch logical chunk (l%16) ^ g(row).
+// ---------------------------------------------------------------------------
+// 16 bytes per lane from (wave-uniform base + this lane's 32-bit offset) to
+// (wave-uniform LDS address + 16 * lane).  Written as asm so that the address
+// stays "SGPR pair + one VGPR" instead of a 64-bit pointer per lane.
+__device__ __forceinline__ void dma16(const char* uniform_base, uint32_t lane_off, uint32_t lds_dst) {
+  asm volatile(
+      "s_mov_b32 m0, %2\n\t"
+      "s_nop 0\n\t"
+      "global_load_lds_dwordx4 %0, %1"
+      :
+      : "v"(lane_off), "s"(uniform_base), "s"(lds_dst)
+      : "memory");
 }
 
-// full tile: every row is valid, addresses are tile base + precomputed offsets
-__device__ __forceinline__ void load_tile_dma(const LoaderOffsets& o, const char* ktile, const char* vtile,
-                                              lds_char* stage, int wave_u) {
+// One 64-key tile of K or of V.  `off` holds this lane's four byte offsets
+// from the tile's first key row.  The last, partial tile redirects rows at or
+// past the valid length to the last valid key (their scores are masked), so
+// nothing outside the rows the caller declared valid is read.
+__device__ __forceinline__ void issue_matrix_tile(const char* base, uint32_t tok_bytes, const uint32_t (&off)[4],
+                                                  int key0, int seq, uint32_t lds_dst, int wave_u, int lane) {
+  const char* tile = base + (int64_t)key0 * tok_bytes;      // wave-uniform
+  if (key0 + kKTile <= seq) {
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    dma16(ktile + o.k[j], stage + (wave_u * 4 + j) * 1024);
-    dma16(vtile + o.v[j], stage + kTileBytes + (wave_u * 4 + j) * 1024);
+    for (int j = 0; j < 4; ++j) dma16(tile, off[j], lds_dst + (wave_u * 4 + j) * 1024);
+  } else {
+    const int last_rel = seq - 1 - key0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int r = 4 * (wave_u * 4 + j) + (lane >> 4);
+      const int rr = r < last_rel ? r : last_rel;
+      const uint32_t o = (uint32_t)rr * tok_bytes + (uint32_t)(((lane & 15) ^ swz(r)) << 4);
+      dma16(tile, o, lds_dst + (wave_u * 4 + j) * 1024);
+    }
   }
 }
 
-// last, partial tile: rows at or past the valid length are redirected to the
-// last valid key (their scores are masked), so nothing outside the rows the
-// caller declared valid is read.
-__device__ __forceinline__ void load_tile_dma_tail(const char* kbase, const char* vbase, int64_t k_tok_bytes,
-                                                   int64_t v_tok_bytes, int key0, int last_key,
-                                                   lds_char* stage, int wave_u, int lane) {
+// The compiler does not know that the asm MFMAs are still in flight when the
+// asm statement retires, so wherever code it generates may touch S or O right
+// after a slot (register moves at control-flow joins, the epilogue) the matrix
+// pipe is drained first: an 8-pass MFMA needs 18 wait states before its result
+// may be read.  The tag makes every use textually distinct, otherwise identical
+// drains at the ends of sibling branches are merged into one AFTER the join,
+// behind the very moves they are meant to precede.
+template <int kTag>
+__device__ __forceinline__ void mfma_drain(f32x16 (&oacc)[kQB][4], f32x16 (&s)[2][kQB]) {
+  asm volatile("s_nop 15\n\ts_nop 15 ; matrix pipe drained, site %12"
+               : "+a"(oacc[0][0]), "+a"(oacc[0][1]), "+a"(oacc[0][2]), "+a"(oacc[0][3]), "+a"(oacc[1][0]),
+                 "+a"(oacc[1][1]), "+a"(oacc[1][2]), "+a"(oacc[1][3]), "+v"(s[0][0]), "+v"(s[0][1]),
+                 "+v"(s[1][0]), "+v"(s[1][1])
+               : "n"(kTag));
+}
+
+struct LaneConst {
+  uint32_t k_addr[8];     // K fragment of d-step ks: key row lane%32 of a 32-key block
+  uint32_t v_addr[4][2];  // V^T fragment of d block db, key sub-quad j, within a 16-key step
+  float c2;               // softmax scale * log2(e)
+  int hf;                 // lane / 32
+};
+
+__device__ __forceinline__ void mask_block(f32x16& s, int key0, int seq, int hf) {
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int r = 4 * (wave_u * 4 + j) + (lane >> 4);
-    int key = key0 + r;
-    key = key < last_key ? key : last_key;
-    const int chunk = (lane & 15) ^ swz(r);
-    dma16(kbase + key * k_tok_bytes + chunk * 16, stage + (wave_u * 4 + j) * 1024);
-    dma16(vbase + key * v_tok_bytes + chunk * 16, stage + kTileBytes + (wave_u * 4 + j) * 1024);
+  for (int i = 0; i < 16; ++i) {
+    const int key = key0 + 8 * (i >> 2) + 4 * hf + (i & 3);
+    if (key >= seq) s[i] = -INFINITY;
   }
 }
 
-__device__ __forceinline__ void wait_vmem_and_sync() {
-  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wave's DMA has landed
-  __syncthreads();
-}
+// ---------------------------------------------------------------------------
+// One pipeline slot of the fast pass.  Keys advance in blocks of 32; block j
+// goes through
+//   S(j)  = K_j Q^T            8 K fragments x 2 query blocks = 16 MFMAs
+//   SM(j) = exp2(scale * S)    VALU only, 2 x 16 scores per lane
+//   PV(j) = O^T += V_j^T P_j^T 8 V fragments x 2 query blocks = 16 MFMAs
+// and slot j runs S(j+1), SM(j) and PV(j-1) together: MFMAs of the two
+// products alternate (no accumulator is touched twice in a row) and the
+// softmax instructions of block j are dealt out between them, so the matrix
+// pipe and the vector ALU of the wave work at the same time.  S(j) lives in
+// s[j&1], P(j) in p[j&1]; with the slot parity a template argument this is
+// pure register naming.
+// ---------------------------------------------------------------------------
+template <int kPar, int kKOff, int kVOff, bool kDoS, bool kDoPV, bool kDoSM>
+__device__ __forceinline__ void slot(const LaneConst& c, const bf16x8 (&qf)[kQB][8], f32x16 (&s)[2][kQB],
+                                     u32x4 (&p)[2][kQB][2], f32x16 (&oacc)[kQB][4], float (&l)[kQB],
+                                     int key0, int key_end) {
+#ifndef SDV2_AHEAD
+#define SDV2_AHEAD 2
+#endif
+  constexpr int kAhead = SDV2_AHEAD;   // fragment pairs are requested this many groups early
+  u32x4 kfrag[8], vfrag[8];
+  f32x16 (&s_cur)[kQB] = s[kPar];
+  f32x16 (&s_nxt)[kQB] = s[kPar ^ 1];
 
-struct SoftmaxState {
-  float m;   // running max of the raw scores of this lane's query
-  float l;   // this lane's share of the running sum
-};
-
-// One 64-key tile from LDS stage `kBuf` (compile-time, so every LDS address is
-// register + immediate).
-template <int kBuf>
-__device__ __forceinline__ void process_tile(const uint32_t (&k_addr)[8], const uint32_t (&v_addr)[4][2],
-                                             const bf16x8 (&qf)[8], f32x16 (&oacc)[4], SoftmaxState& st,
-                                             float c2, int key0, int seq, int hf) {
-  constexpr int kBase = kBuf * kStageBytes;
-  constexpr int vBase = kBuf * kStageBytes + kTileBytes;
-
-  // ---- S^T = K Q^T : two 32-key blocks --------------------------------
-  // 16 MFMAs, the two accumulators alternating; K fragments are fetched from
-  // LDS kAhead MFMAs ahead.  Step s covers d-step s/2 of key block s%2.
-  f32x16 sacc[2];
-#pragma unroll
-  for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.f;
-  constexpr int kAhead = 4;
-  u32x4 kf[16];
-  static_for<kAhead>([&](auto ic) {
-    constexpr int s = decltype(ic)::value;
-    kf[s] = lds_read_b128<kBase + (s & 1) * 32 * 256>(k_addr[s >> 1]);
-  });
-  static_for<16>([&](auto ic) {
-    constexpr int s = decltype(ic)::value;
-    if constexpr (s + kAhead < 16)
-      kf[s + kAhead] = lds_read_b128<kBase + ((s + kAhead) & 1) * 32 * 256>(k_addr[(s + kAhead) >> 1]);
-    wait_lds<(s + kAhead < 16) ? kAhead : 15 - s>(kf[s]);
-    sacc[s & 1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, kf[s]), qf[s >> 1],
-                                                          sacc[s & 1], 0, 0, 0);
-    __builtin_amdgcn_sched_barrier(0);
-  });
-
-  // first V^T fragments: issued now, they land while the softmax runs.
-  // Step s covers key step s/4 (16 keys) and d block s%4.
-  constexpr int vAhead = 4;
-  u32x4 vf[16];
-  auto v_frag = [&](auto ic) {
-    constexpr int s = decltype(ic)::value;
-    constexpr int kk = s >> 2, db = s & 3;
-    const u32x2 lo = lds_read_tr16_b64<vBase + kk * 16 * 256>(v_addr[db][0]);
-    const u32x2 hi = lds_read_tr16_b64<vBase + kk * 16 * 256>(v_addr[db][1]);
-    vf[s] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3);
+  auto request = [&](auto ic) {
+    constexpr int g = decltype(ic)::value;
+    if constexpr (kDoS) kfrag[g] = lds_read_b128<kKOff>(c.k_addr[g]);
+    if constexpr (kDoPV) {
+      constexpr int kk = g >> 2, db = g & 3;
+      const u32x2 lo = lds_read_tr16_b64<kVOff + kk * 16 * 256>(c.v_addr[db][0]);
+      const u32x2 hi = lds_read_tr16_b64<kVOff + kk * 16 * 256>(c.v_addr[db][1]);
+      vfrag[g] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3);
+    }
   };
-  static_for<vAhead>(v_frag);
+  // reads issued after the K (resp. V) fragment of group g, when group g runs
+  constexpr int kPerGroup = (kDoS ? 1 : 0) + (kDoPV ? 2 : 0);
+
+  static_for<kAhead>(request);
+
+  if constexpr (kDoSM) {
+    // the last, partial tile and the padding tiles behind it.  The test value
+    // goes through an empty asm so that the compiler cannot fold this uniform,
+    // rarely taken branch into the per-lane compares and hoist those.
+    int beyond = key0 + 32 - key_end;
+    asm volatile("" : "+s"(beyond));
+    if (beyond > 0) {
+#pragma unroll
+      for (int qb = 0; qb < kQB; ++qb) mask_block(s_cur[qb], key0, key_end, c.hf);
+    }
+  }
   __builtin_amdgcn_sched_barrier(0);
 
-  // ---- mask the tail of the last tile ---------------------------------
-  if (key0 + kKTile > seq) {
-#pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int key = key0 + kb * 32 + 8 * (i >> 2) + 4 * hf + (i & 3);
-        if (key >= seq) sacc[kb][i] = -INFINITY;
+  // A wave issues in order: a vector instruction only overlaps an MFMA if it
+  // follows it in the stream, and it stalls the stream if it needs the result
+  // of the instruction just before it.  So every MFMA is followed by a few
+  // softmax instructions that are independent of each other: the 32 scores of
+  // block j (both query blocks) flow through scale -> exp2 -> pack + row sum
+  // one step apart.  Score t belongs to group g = t/4: query block (t%4)/2,
+  // accumulator register 2g + t%2.
+  float scaled[33], weight[33];
+  auto score = [&](auto tc) -> float {
+    constexpr int t = decltype(tc)::value;
+    return s_cur[(t & 3) >> 1][2 * (t >> 2) + (t & 1)];
+  };
+  auto softmax_step = [&](auto tc) {
+    constexpr int t = decltype(tc)::value;      // 0..33: stage 1 of score t, stage 2 of t-1, stage 3 of t-2
+    if constexpr (kDoSM) {
+      if constexpr (t < 32) {
+        scaled[t] = score(tc) * c.c2;
+        pin(scaled[t]);
       }
-  }
-
-  // ---- online softmax, one query per lane ------------------------------
-  float mloc = sacc[0][0];
-#pragma unroll
-  for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, sacc[kb][i]);
-  mloc = half_max(mloc);
-  const float m_new = fmaxf(st.m, mloc);
-  const float alpha = __builtin_amdgcn_exp2f((st.m - m_new) * c2);
-  const float mc = m_new * c2;
-  st.m = m_new;
-  float psum = 0.f;
-#pragma unroll
-  for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][i], c2, -mc));
-      sacc[kb][i] = p;
-      psum += p;
+      if constexpr (t >= 1 && t - 1 < 32) {
+        weight[t - 1] = __builtin_amdgcn_exp2f(scaled[t - 1]);
+        pin(weight[t - 1]);
+      }
+      if constexpr (t >= 2 && t - 2 < 32 && ((t - 2) & 1) == 1) {
+        constexpr int u = t - 2, g = u >> 2, qb = (u & 3) >> 1;
+        uint32_t packed = pack_bf16x2(weight[u - 1], weight[u]);
+        l[qb] = add_bf16_pair(packed, l[qb]);
+        pin(packed);
+        pin(l[qb]);
+        p[kPar][qb][g >> 2][g & 3] = packed;
+      }
     }
-  st.l = st.l * alpha + psum;
-  if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+  };
+
+  static_for<32>([&](auto tc) {
+    constexpr int t = decltype(tc)::value;
+    constexpr int g = t >> 2, i = t & 3;
+    constexpr int later = (g + kAhead < 8 ? kAhead : 7 - g) * kPerGroup;   // reads of later groups in flight
+    constexpr int kk = g >> 2, db = g & 3;
+    if constexpr (i == 0 && g + kAhead < 8) request(std::integral_constant<int, g + kAhead>{});
+
+    if constexpr (i == 0 && kDoS) {
+      if constexpr (g == 0) mfma_s_first<later + (kDoPV ? 2 : 0)>(s_nxt[0], kfrag[g], qf[0][g]);
+      else mfma_s<later + (kDoPV ? 2 : 0)>(s_nxt[0], kfrag[g], qf[0][g]);
+    }
+    if constexpr (i == 1 && kDoS) {
+      if constexpr (g == 0) mfma_s_first<-1>(s_nxt[1], kfrag[g], qf[1][g]);
+      else mfma_s<-1>(s_nxt[1], kfrag[g], qf[1][g]);
+    }
+    if constexpr (i == 2 && kDoPV) mfma_o<later>(oacc[0][db], vfrag[g], p[kPar ^ 1][0][kk]);
+    if constexpr (i == 3 && kDoPV) mfma_o<-1>(oacc[1][db], vfrag[g], p[kPar ^ 1][1][kk]);
+
+    softmax_step(tc);
+    __builtin_amdgcn_sched_barrier(0);
+  });
+  softmax_step(std::integral_constant<int, 32>{});
+  softmax_step(std::integral_constant<int, 33>{});
+}
+
+// ---------------------------------------------------------------------------
+// Exact pass: conventional online softmax with a running maximum, one 64-key
+// tile at a time, nothing overlapped.  Only reached when the fast pass saw a
+// row sum leave the safe range, so its speed does not matter.
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void exact_pass(const AttnKernelArgs& a, const LaneConst& c, const bf16x8 (&qf)[kQB][8],
+                                        f32x16 (&oacc)[kQB][4], float (&m_run)[kQB], float (&l_run)[kQB],
+                                        const char* kbase, const char* vbase, uint32_t k_tok_bytes,
+                                        uint32_t v_tok_bytes, const uint32_t (&k_ld)[4], const uint32_t (&v_ld)[4],
+                                        int tile_begin, int n, int seq, uint32_t lds_addr0, lds_char* lds,
+                                        int wave_u, int lane) {
+#pragma unroll
+  for (int qb = 0; qb < kQB; ++qb) {
+    m_run[qb] = -INFINITY;
+    l_run[qb] = 0.f;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
+      for (int i = 0; i < 16; ++i) oacc[qb][db][i] = 0.f;
   }
-
-  // ---- P^T as the B operand: accumulator registers 8*step..8*step+7 ----
-  bf16x8 pf[2][2];
+  for (int T = 0; T < n; ++T) {
+    const int key0 = (tile_begin + T) * kKTile;
+    __syncthreads();     // everyone is done with the previous tile
+    issue_matrix_tile(kbase, k_tok_bytes, k_ld, key0, seq, lds_addr0 + kLdsK(0), wave_u, lane);
+    issue_matrix_tile(vbase, v_tok_bytes, v_ld, key0, seq, lds_addr0 + kLdsV(0), wave_u, lane);
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
 #pragma unroll
-  for (int kb = 0; kb < 2; ++kb)
+    for (int qb = 0; qb < kQB; ++qb) {
+      f32x16 sacc[2];
 #pragma unroll
-    for (int s2 = 0; s2 < 2; ++s2) {
-      union { uint32_t u[4]; bf16x8 v; } pk;
+      for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        pk.u[j] = pack_bf16x2(sacc[kb][8 * s2 + 2 * j], sacc[kb][8 * s2 + 2 * j + 1]);
-      pf[kb][s2] = pk.v;
+        for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) {
+          const bf16x8 kf = *reinterpret_cast<__attribute__((address_space(3))) const bf16x8*>(
+              lds + (c.k_addr[ks] - lds_addr0) + kLdsK(0) + kb * 32 * 256);
+          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][ks], sacc[kb], 0, 0, 0);
+        }
+        if (key0 + kb * 32 + 32 > seq) mask_block(sacc[kb], key0 + kb * 32, seq, c.hf);
+      }
+      float mloc = sacc[0][0];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, sacc[kb][i]);
+      mloc = half_max(mloc);
+      const float m_new = fmaxf(m_run[qb], mloc);      // finite: every tile has a valid key
+      const float alpha = __builtin_amdgcn_exp2f((m_run[qb] - m_new) * c.c2);
+      const float mc = m_new * c.c2;
+      m_run[qb] = m_new;
+      float psum = 0.f;
+      bf16x8 pf[2][2];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+          union { uint32_t u[4]; bf16x8 v; } pk;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][8 * st + 2 * j], c.c2, -mc));
+            const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[kb][8 * st + 2 * j + 1], c.c2, -mc));
+            psum += p0 + p1;
+            pk.u[j] = pack_bf16x2(p0, p1);
+          }
+          pf[kb][st] = pk.v;
+        }
+      l_run[qb] = l_run[qb] * alpha + psum;
+#pragma unroll
+      for (int db = 0; db < 4; ++db) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[qb][db][i] *= alpha;
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(
+              lds + (c.v_addr[db][0] - lds_addr0) + kk * 16 * 256));
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(
+              lds + (c.v_addr[db][1] - lds_addr0) + kk * 16 * 256));
+          const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          oacc[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both),
+                                                                 pf[kk >> 1][kk & 1], oacc[qb][db], 0, 0, 0);
+        }
+      }
     }
-
-  // ---- O^T += V^T P^T ----------------------------------------------------
-  __builtin_amdgcn_sched_barrier(0);
-  static_for<16>([&](auto ic) {
-    constexpr int s = decltype(ic)::value;
-    if constexpr (s + vAhead < 16) v_frag(std::integral_constant<int, s + vAhead>{});
-    wait_lds<(s + vAhead < 16) ? 2 * vAhead : 2 * (15 - s)>(vf[s]);
-    constexpr int kk = s >> 2, db = s & 3;
-    oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, vf[s]), pf[kk >> 1][kk & 1],
-                                                       oacc[db], 0, 0, 0);
-    __builtin_amdgcn_sched_barrier(0);
-  });
+  }
 }
 
-__global__ __launch_bounds__(kThreads, 2)
+__global__ __launch_bounds__(kThreads, 1)
 void swa_attn_fwd_kernel(const AttnKernelArgs a) {
-  __shared__ __attribute__((aligned(1024))) char smem[2 * kStageBytes];
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
   lds_char* lds = (lds_char*)smem;
 
   const int tid = threadIdx.x;
@@ -297,10 +474,27 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   const int wave = tid >> 6;
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int hf = lane >> 5;                 // which half of the wave
-  const int qtile = blockIdx.x;
-  const int head = blockIdx.y;
-  const int row = blockIdx.z / a.num_splits;
-  const int split = blockIdx.z - row * a.num_splits;
+  // Workgroups are dealt to the eight XCDs round robin by id, and each XCD has
+  // its own L2.  Work items are ordered so that the query tiles of one (row,
+  // head, key split) are neighbours, and XCD x takes the x-th eighth of that
+  // list: the workgroups that stream the same K / V run on the same XCD at the
+  // same time and all but the first fetch of a tile hit in L2.
+  int qtile, head, row, split;
+  {
+    const int nq = (a.q_tokens + kQTile - 1) / kQTile;
+    const int total = nq * a.heads * a.rows * a.num_splits;
+    const int xcd = blockIdx.x & 7;
+    const int first = (int)(((int64_t)xcd * total) >> 3);
+    const int end = (int)(((int64_t)(xcd + 1) * total) >> 3);
+    int item = first + (blockIdx.x >> 3);
+    if (item >= end) return;
+    qtile = item % nq;
+    item /= nq;
+    split = item % a.num_splits;
+    item /= a.num_splits;
+    head = item % a.heads;
+    row = item / a.heads;
+  }
 
   int seq = a.seq_lens ? a.seq_lens[row] : a.max_seq_len;
   seq = seq < a.max_seq_len ? seq : a.max_seq_len;
@@ -310,55 +504,68 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   const int tile_begin = split * per_split;
   int tile_end = tile_begin + per_split;
   tile_end = tile_end < ntiles ? tile_end : ntiles;
+  const int n = tile_end - tile_begin;       // tiles this workgroup streams
 
+  const uint32_t lds_addr0 = (uint32_t)(uintptr_t)lds;
   const char* kbase = reinterpret_cast<const char*>(a.k + row * a.k_st.row + head * a.k_st.head);
   const char* vbase = reinterpret_cast<const char*>(a.v + row * a.v_st.row + head * a.v_st.head);
-  const int64_t k_tok_bytes = a.k_st.token * 2;
-  const int64_t v_tok_bytes = a.v_st.token * 2;
+  const uint32_t k_tok_bytes = (uint32_t)(a.k_st.token * 2);
+  const uint32_t v_tok_bytes = (uint32_t)(a.v_st.token * 2);
 
-  LoaderOffsets lo;
+  uint32_t k_ld[4], v_ld[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int r = 4 * (wave * 4 + j) + (lane >> 4);
     const int chunk = (lane & 15) ^ swz(r);
-    lo.k[j] = (uint32_t)(r * k_tok_bytes + chunk * 16);
-    lo.v[j] = (uint32_t)(r * v_tok_bytes + chunk * 16);
+    k_ld[j] = (uint32_t)(r * k_tok_bytes + chunk * 16);
+    v_ld[j] = (uint32_t)(r * v_tok_bytes + chunk * 16);
   }
-
-  auto issue_tile = [&](int t, int buf) {
-    const int key0 = t * kKTile;
-    lds_char* stage = lds + buf * kStageBytes;
-    if (key0 + kKTile <= seq)
-      load_tile_dma(lo, kbase + key0 * k_tok_bytes, vbase + key0 * v_tok_bytes, stage, wave_u);
-    else
-      load_tile_dma_tail(kbase, vbase, k_tok_bytes, v_tok_bytes, key0, seq - 1, stage, wave_u, lane);
+  // T is the tile index inside this workgroup's range
+  auto issue_k = [&](int T, int buf) {
+    issue_matrix_tile(kbase, k_tok_bytes, k_ld, (tile_begin + T) * kKTile, seq, lds_addr0 + kLdsK(buf), wave_u, lane);
+  };
+  auto issue_v = [&](int T, int buf) {
+    issue_matrix_tile(vbase, v_tok_bytes, v_ld, (tile_begin + T) * kKTile, seq, lds_addr0 + kLdsV(buf), wave_u, lane);
   };
 
-  if (tile_begin < tile_end) issue_tile(tile_begin, 0);
+  if (n > 0) {
+    // Every buffer starts with real (finite) data, also those whose tile does
+    // not exist: they are only ever met by all-zero weights.
+    issue_k(0, 0);
+    issue_v(0, 0);
+    issue_k(n > 1 ? 1 : n - 1, 1);
+    issue_v(n > 1 ? 1 : n - 1, 1);
+    issue_k(n > 2 ? 2 : n - 1, 2);
+    issue_v(0, 2);              // stand-in for "V tile -1", met by the all-zero P(-1)
+  }
 
-  // ---- this lane's query row, as the B operand of S^T = K Q^T -------------
-  const int q_row = qtile * kQTile + wave * kQRowsPerWave + (lane & 31);
-  const int q_row_c = q_row < a.q_tokens ? q_row : a.q_tokens - 1;
-  const uint16_t* qp = a.q + row * a.q_st.row + (int64_t)q_row_c * a.q_st.token + head * a.q_st.head + 8 * hf;
-  bf16x8 qf[8];
+  // ---- this lane's query rows, as the B operand of S^T = K Q^T -------------
+  int q_row[kQB];
+  bf16x8 qf[kQB][8];
 #pragma unroll
-  for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
+  for (int qb = 0; qb < kQB; ++qb) {
+    q_row[qb] = qtile * kQTile + wave * kQRowsPerWave + qb * 32 + (lane & 31);
+    const int q_row_c = q_row[qb] < a.q_tokens ? q_row[qb] : a.q_tokens - 1;
+    const uint16_t* qp = a.q + row * a.q_st.row + (int64_t)q_row_c * a.q_st.token + head * a.q_st.head + 8 * hf;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qf[qb][ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
+  }
 
-  // ---- per-lane LDS read offsets -------------------------------------------
-  // K (A operand): key = kb*32 + lane%32, chunk = 2*ks + hf
-  const uint32_t lds_addr0 = (uint32_t)(uintptr_t)lds;
-  uint32_t k_addr[8];
+  // ---- per-lane LDS read addresses ------------------------------------------
+  LaneConst c;
+  c.c2 = a.scale_log2;
+  c.hf = hf;
   {
+    // K (A operand): key = lane%32 of the block, chunk = 2*ks + hf
     const int r = lane & 31;
     const int base = r * 256 + ((hf ^ swz(r)) << 4);
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) k_addr[ks] = lds_addr0 + (uint32_t)(base ^ (ks << 5));
+    for (int ks = 0; ks < 8; ++ks) c.k_addr[ks] = lds_addr0 + (uint32_t)(base ^ (ks << 5));
   }
-  // V^T (A operand) through the transposing read: in each group of 16 lanes,
-  // lane i supplies the address of key (i / 4), 8 bytes at d-offset 4 * (i % 4);
-  // it receives d = i, keys 0..3.  Group = (hf, dhalf).
-  uint32_t v_addr[4][2];
   {
+    // V^T (A operand) through the transposing read: in each group of 16 lanes,
+    // lane i supplies the address of key (i / 4), 8 bytes at d-offset 4 * (i % 4);
+    // it receives d = i, keys 0..3.  Group = (hf, dhalf).  Relative to V buffer 0.
     const int i16 = lane & 15;
     const int dhalf = (lane >> 4) & 1;
     const int krow = i16 >> 2;
@@ -367,67 +574,133 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int r = 8 * j + 4 * hf + krow;                 // + 16 * kk added as an immediate
-        const int c = db * 4 + dhalf * 2 + ((i16 & 3) >> 1);
-        v_addr[db][j] = lds_addr0 + (uint32_t)(r * 256 + ((c ^ swz(r)) << 4) + (i16 & 1) * 8);
+        const int ch = db * 4 + dhalf * 2 + ((i16 & 3) >> 1);
+        c.v_addr[db][j] = lds_addr0 + kLdsVBase + (uint32_t)(r * 256 + ((ch ^ swz(r)) << 4) + (i16 & 1) * 8);
       }
   }
 
-  f32x16 oacc[4];
+  f32x16 oacc[kQB][4];
 #pragma unroll
-  for (int db = 0; db < 4; ++db)
+  for (int qb = 0; qb < kQB; ++qb)
 #pragma unroll
-    for (int i = 0; i < 16; ++i) oacc[db][i] = 0.f;
-  SoftmaxState st{-INFINITY, 0.f};
-  const float c2 = a.scale_log2;
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) oacc[qb][db][i] = 0.f;
+  f32x16 s[2][kQB];
+  u32x4 p[2][kQB][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int qb = 0; qb < kQB; ++qb)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) p[i][qb][j] = u32x4{0u, 0u, 0u, 0u};
+  float l_run[kQB] = {0.f, 0.f};     // this lane's share of each block's row sum
+  float m_run[kQB] = {0.f, 0.f};     // reference of the exponent: 0 in the fast pass
+  bool unsafe = false;
 
-  wait_vmem_and_sync();   // first tile and the Q fragments have arrived
+  // Tile T (64 keys) = blocks 2T, 2T+1, in K / V buffers T % 3.  Slot 2T needs
+  // K tile T (second half) and V tile T-1 (second half); slot 2T+1 needs K tile
+  // T+1 (first half) and V tile T (first half).  After slot 2T the buffers of
+  // K tile T and V tile T-1 are free: that is where the one barrier per tile
+  // sits, followed by the requests for K tile T+3 and V tile T+2.  What the
+  // next two slots read was requested two barriers earlier, so the wait before
+  // the barrier leaves the newest eight transfers in flight.
+  //
+  // Every tile runs the same code and the loop body is three whole tiles with
+  // a single way in and out, so the accumulators keep their registers from trip
+  // to trip (the compiler must never be given a reason to move them while asm
+  // MFMAs are in flight).  The tile count is padded to a multiple of three:
+  // padding tiles, like the tail of a partial tile, have all their scores
+  // masked to -inf, so their weights are exact zeros against whatever finite
+  // data the buffers still hold.  In the first slot P(-1) is zero likewise.
+  const int key_end = seq < tile_end * kKTile ? seq : tile_end * kKTile;
+  auto row_sums_unsafe = [&]() {
+    bool bad = false;
+#pragma unroll
+    for (int qb = 0; qb < kQB; ++qb) bad |= !(l_run[qb] >= 0x1p-100f && l_run[qb] <= 0x1p100f);
+    return __builtin_amdgcn_ballot_w64(bad) != 0;
+  };
+  auto do_tile = [&](auto buf_c, int T) {
+    constexpr int kB = decltype(buf_c)::value;              // T % 3
+    constexpr int kBNext = (kB + 1) % kStages, kBPrev = (kB + 2) % kStages;
+    const int key0 = (tile_begin + T) * kKTile;
+    slot<0, kLdsK(kB) + 32 * 256, kLdsVRel(kBPrev) + 32 * 256, true, true, true>(c, qf, s, p, oacc, l_run, key0,
+                                                                                key_end);
+    if (T + 3 < n) {
+      __builtin_amdgcn_s_waitcnt(0x0F78);   // vmcnt(8)
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+    }
+    __syncthreads();
+    if (T + 3 < n) issue_k(T + 3, kB);
+    if (T + 2 < n) issue_v(T + 2, kBPrev);
+    slot<1, kLdsK(kBNext), kLdsVRel(kB), true, true, true>(c, qf, s, p, oacc, l_run, key0 + 32, key_end);
+    if (T < n) unsafe |= row_sums_unsafe();
+  };
+  using B0 = std::integral_constant<int, 0>;
+  using B1 = std::integral_constant<int, 1>;
+  using B2 = std::integral_constant<int, 2>;
 
-  // Two tiles per trip so the LDS stage is a compile-time constant.
-  for (int t = tile_begin; t < tile_end; t += 2) {
-    if (t + 1 < tile_end) issue_tile(t + 1, 1);
-    process_tile<0>(k_addr, v_addr, qf, oacc, st, c2, t * kKTile, seq, hf);
-    wait_vmem_and_sync();
-    if (t + 1 >= tile_end) break;
-    if (t + 2 < tile_end) issue_tile(t + 2, 0);
-    process_tile<1>(k_addr, v_addr, qf, oacc, st, c2, (t + 1) * kKTile, seq, hf);
-    wait_vmem_and_sync();
+  if (n > 0) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();        // the first tiles and the Q fragments have arrived
+    // S(0) alone fills the pipeline
+    slot<1, kLdsK(0), 0, true, false, false>(c, qf, s, p, oacc, l_run, 0, key_end);
+    for (int T = 0; T < n; T += 3) {
+      do_tile(B0{}, T);
+      do_tile(B1{}, T + 1);
+      do_tile(B2{}, T + 2);
+    }
+    // PV of the last block (odd -> p[1], second half of the tile in V buffer 2) empties the pipeline
+    slot<0, 0, kLdsVRel(2) + 32 * 256, false, true, false>(c, qf, s, p, oacc, l_run, 0, key_end);
+    mfma_drain<0>(oacc, s);
+
+    // Did any wave of the workgroup see an unsafe row sum?  (LDS is free now.)
+    __syncthreads();
+    if (tid == 0) *reinterpret_cast<__attribute__((address_space(3))) int*>(lds) = 0;
+    __syncthreads();
+    if (unsafe && lane == 0) *reinterpret_cast<__attribute__((address_space(3))) int*>(lds) = 1;
+    __syncthreads();
+    const int redo = *reinterpret_cast<__attribute__((address_space(3))) int*>(lds);
+    if (redo)
+      exact_pass(a, c, qf, oacc, m_run, l_run, kbase, vbase, k_tok_bytes, v_tok_bytes, k_ld, v_ld, tile_begin, n,
+                 seq, lds_addr0, lds, wave_u, lane);
   }
-
-  float m_run = st.m;
-  float l_run = st.l;
 
   // ---- epilogue ---------------------------------------------------------------
-  const float l_tot = half_sum(l_run);
-  const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-  if (q_row >= a.q_tokens) return;
-
-  if (a.num_splits == 1) {
-    uint16_t* op = a.out + row * a.o_st.row + (int64_t)q_row * a.o_st.token + head * a.o_st.head;
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+  for (int qb = 0; qb < kQB; ++qb) {
+    const float l_tot = half_sum(l_run[qb]);
+    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+    if (q_row[qb] >= a.q_tokens) continue;
+    if (a.num_splits == 1) {
+      uint16_t* op = a.out + row * a.o_st.row + (int64_t)q_row[qb] * a.o_st.token + head * a.o_st.head;
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        uint2 w;
-        w.x = pack_bf16x2(oacc[db][4 * g] * inv, oacc[db][4 * g + 1] * inv);
-        w.y = pack_bf16x2(oacc[db][4 * g + 2] * inv, oacc[db][4 * g + 3] * inv);
-        *reinterpret_cast<uint2*>(op + db * 32 + 8 * g + 4 * hf) = w;
-      }
-  } else {
-    const int64_t prow = (((int64_t)split * a.rows + row) * a.heads + head) * a.q_tokens + q_row;
-    float* po = a.part_o + prow * kD;
+      for (int db = 0; db < 4; ++db)
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
+        for (int g = 0; g < 4; ++g) {
+          uint2 w;
+          w.x = pack_bf16x2(oacc[qb][db][4 * g] * inv, oacc[qb][db][4 * g + 1] * inv);
+          w.y = pack_bf16x2(oacc[qb][db][4 * g + 2] * inv, oacc[qb][db][4 * g + 3] * inv);
+          *reinterpret_cast<uint2*>(op + db * 32 + 8 * g + 4 * hf) = w;
+        }
+    } else {
+      const int64_t prow = (((int64_t)split * a.rows + row) * a.heads + head) * a.q_tokens + q_row[qb];
+      float* po = a.part_o + prow * kD;
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        float4 w;
-        w.x = oacc[db][4 * g] * inv;
-        w.y = oacc[db][4 * g + 1] * inv;
-        w.z = oacc[db][4 * g + 2] * inv;
-        w.w = oacc[db][4 * g + 3] * inv;
-        *reinterpret_cast<float4*>(po + db * 32 + 8 * g + 4 * hf) = w;
-      }
-    if (hf == 0)
-      a.part_lse[prow] = l_tot > 0.f ? m_run * c2 + __builtin_amdgcn_logf(l_tot) : -INFINITY;
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          float4 w;
+          w.x = oacc[qb][db][4 * g] * inv;
+          w.y = oacc[qb][db][4 * g + 1] * inv;
+          w.z = oacc[qb][db][4 * g + 2] * inv;
+          w.w = oacc[qb][db][4 * g + 3] * inv;
+          *reinterpret_cast<float4*>(po + db * 32 + 8 * g + 4 * hf) = w;
+        }
+      if (hf == 0)
+        a.part_lse[prow] = l_tot > 0.f ? m_run[qb] * c.c2 + __builtin_amdgcn_logf(l_tot) : -INFINITY;
+    }
   }
 }
 
@@ -475,15 +748,20 @@ size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 extern "C" int sdv2_swa_attn_default_splits(int32_t rows, int32_t q_tokens, int32_t heads, int32_t max_seq_len) {
   if (rows <= 0 || q_tokens <= 0 || heads <= 0 || max_seq_len <= 0) return 1;
-  // 256 CUs x 2 resident workgroups
-  const int64_t slots = 512;
+  // One workgroup per CU.  With s key-range splits there are qwork * s
+  // workgroups of 1/s of the keys each: time ~ ceil(qwork * s / 256) / s rounds,
+  // plus a small charge per split for writing and merging partial results.
   const int64_t qwork = (int64_t)rows * heads * ((q_tokens + kQTile - 1) / kQTile);
   const int ntiles = (max_seq_len + kKTile - 1) / kKTile;
-  int64_t splits = slots / qwork;
-  if (splits < 1) splits = 1;
-  if (splits > 8) splits = 8;
-  if (splits > ntiles / 8) splits = ntiles / 8 > 0 ? ntiles / 8 : 1;
-  return (int)splits;
+  int best = 1;
+  double best_cost = 1e30;
+  for (int sp = 1; sp <= 8; ++sp) {
+    if (sp > 1 && ntiles / sp < 8) break;
+    const int64_t rounds = (qwork * sp + kCuSlots - 1) / kCuSlots;
+    const double cost = (double)rounds / sp * (1.0 + 0.02 * (sp - 1));
+    if (cost < best_cost - 1e-9) { best_cost = cost; best = sp; }
+  }
+  return best;
 }
 
 extern "C" size_t sdv2_swa_attn_workspace_bytes(int32_t rows, int32_t q_tokens, int32_t heads,
@@ -537,9 +815,15 @@ extern "C" int sdv2_swa_attn_fwd(const sdv2_attn_params* p) {
   }
 
   hipStream_t stream = static_cast<hipStream_t>(p->stream);
-  dim3 grid((p->q_tokens + kQTile - 1) / kQTile, p->heads, p->rows * splits);
+  const int64_t items = (int64_t)((p->q_tokens + kQTile - 1) / kQTile) * p->heads * p->rows * splits;
+  if (items > (1 << 28)) return SDV2_ERR_INVALID_ARG;
+  dim3 grid((unsigned)(8 * ((items + 7) / 8)));
   if (p->stages != SDV2_STAGE_MERGE) {
-    hipLaunchKernelGGL(swa_attn_fwd_kernel, grid, dim3(kThreads), 0, stream, a);
+    // 96 KB of LDS is more than the static limit: ask for it once per process
+    static const hipError_t lds_attr = hipFuncSetAttribute(
+        reinterpret_cast<const void*>(swa_attn_fwd_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    if (lds_attr != hipSuccess) return SDV2_ERR_LAUNCH;
+    hipLaunchKernelGGL(swa_attn_fwd_kernel, grid, dim3(kThreads), kLdsBytes, stream, a);
     if (hipGetLastError() != hipSuccess) return SDV2_ERR_LAUNCH;
   }
   if (splits > 1 && p->stages != SDV2_STAGE_PARTIAL) {

@@ -48,3 +48,46 @@ def test_attention_matches_fp32_oracle(gpu_device, rows, S, H, L, seq, head_majo
     got = ops.swa_attention(q.to(gpu_device), kd, vd, sl, num_splits=splits)
     torch.cuda.synchronize()
     _check(got.cpu(), want)
+
+
+@pytest.mark.parametrize("kind", ["huge_positive", "huge_negative", "mixed_rows"])
+@pytest.mark.parametrize("splits", [1, 2])
+def test_attention_exact_fallback_on_extreme_scores(gpu_device, kind, splits):
+    """Scaled scores far outside +-100 (log2 units) leave the range in which
+    exp2 without a running maximum is representable; the kernel must notice and
+    recompute with the running-maximum recurrence."""
+    from streamdiffusionv2_amd import ops
+
+    torch.manual_seed(5)
+    rows, S, H, L = 1, 300, 2, 700
+    q = torch.randn(rows, S, H, 128)
+    k = torch.randn(rows, L, H, 128)
+    v = torch.randn(rows, L, H, 128)
+    w = torch.randn(128)
+    w = w / w.norm()
+    if kind == "huge_positive":
+        q, k = q * 14.0, k * 14.0                      # |scaled score| up to several hundred
+    elif kind == "huge_negative":
+        q = q + 40.0 * w                               # every score about -40*40 / sqrt(128) ~ -141 nat
+        k = k - 40.0 * w
+    else:
+        q[:, 150:] = q[:, 150:] * 20.0                 # only some query rows are extreme
+    q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+    want = oracle.attention_fp32_reference(q, k, v, [L] * rows)
+    got = ops.swa_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), None, num_splits=splits)
+    torch.cuda.synchronize()
+    _check(got.cpu(), want)
+
+
+def test_attention_tiny_sequences(gpu_device):
+    from streamdiffusionv2_amd import ops
+
+    torch.manual_seed(6)
+    for L in (1, 2, 5, 31, 33, 64, 65):
+        q = torch.randn(1, 40, 1, 128).bfloat16()
+        k = torch.randn(1, L, 1, 128).bfloat16()
+        v = torch.randn(1, L, 1, 128).bfloat16()
+        want = oracle.attention_fp32_reference(q, k, v, [L])
+        got = ops.swa_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), None)
+        torch.cuda.synchronize()
+        _check(got.cpu(), want)
