@@ -749,16 +749,22 @@ size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 extern "C" int sdv2_swa_attn_default_splits(int32_t rows, int32_t q_tokens, int32_t heads, int32_t max_seq_len) {
   if (rows <= 0 || q_tokens <= 0 || heads <= 0 || max_seq_len <= 0) return 1;
   // One workgroup per CU.  With s key-range splits there are qwork * s
-  // workgroups of 1/s of the keys each: time ~ ceil(qwork * s / 256) / s rounds,
-  // plus a small charge per split for writing and merging partial results.
+  // workgroups; they run in ceil(qwork * s / 256) rounds, each as long as one
+  // workgroup's tile count (padded to a multiple of three) plus a fixed start /
+  // end cost of about three tile times.  Writing and merging the fp32 partial
+  // results costs roughly one tile time per 7 MB per split.  Constants fitted
+  // to measurements on the five benchmark shapes.
   const int64_t qwork = (int64_t)rows * heads * ((q_tokens + kQTile - 1) / kQTile);
   const int ntiles = (max_seq_len + kKTile - 1) / kKTile;
+  const double partial_tiles = (double)rows * heads * q_tokens * kD * 4 / 7.0e6;
   int best = 1;
-  double best_cost = 1e30;
+  double best_cost = 1e300;
   for (int sp = 1; sp <= 8; ++sp) {
-    if (sp > 1 && ntiles / sp < 8) break;
+    const int per = (ntiles + sp - 1) / sp;
+    if (sp > 1 && per < 6) break;
     const int64_t rounds = (qwork * sp + kCuSlots - 1) / kCuSlots;
-    const double cost = (double)rounds / sp * (1.0 + 0.02 * (sp - 1));
+    const int padded = (per + 2) / 3 * 3;
+    const double cost = (double)rounds * (padded + 3) + (sp > 1 ? sp * partial_tiles : 0.0);
     if (cost < best_cost - 1e-9) { best_cost = cost; best = sp; }
   }
   return best;

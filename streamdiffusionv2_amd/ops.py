@@ -45,6 +45,10 @@ def _stream_ptr(dev: torch.device) -> int:
     return torch.cuda.current_stream(dev).cuda_stream
 
 
+def _current_device_index() -> int:
+    return torch.cuda.current_device()
+
+
 def _i64_array(values: Sequence[int]):
     return (C.c_int64 * len(values))(*[int(v) for v in values])
 
@@ -222,6 +226,138 @@ def swa_attention(
     with torch.cuda.device(dev):
         _capi.check(lib.sdv2_swa_attn_fwd(C.byref(p)), "sdv2_swa_attn_fwd")
     return out
+
+
+class LayerLauncher:
+    """Pre-built launch descriptors for one layer's (append, attention) pair.
+
+    A chunk step calls the path once per transformer block, every time with the
+    same cache, shapes and strides; only the slot, the RoPE frame, the index
+    values and the q/k/v pointers change.  Building the two C structs from
+    scratch costs more host time than the kernels take on the GPU, so they are
+    built once per (cache, shape) and patched per call.
+    """
+
+    @staticmethod
+    def _sig(t):
+        return (tuple(t.shape), tuple(t.stride()), t.dtype)
+
+    def __init__(self, k_cache, v_cache, global_end_index, local_end_index, freqs_table, grid, q_like, k_like=None,
+                 v_like=None):
+        k_like = q_like if k_like is None else k_like
+        v_like = q_like if v_like is None else v_like
+        rows, tokens, heads, _ = q_like.shape
+        if tuple(k_like.shape) != tuple(q_like.shape) or tuple(v_like.shape) != tuple(q_like.shape):
+            raise RuntimeError("q, k and v must have one shape")
+        if rows > _capi.MAX_ROWS:
+            raise RuntimeError(f"LayerLauncher handles at most {_capi.MAX_ROWS} rows")
+        if q_like.dtype != torch.bfloat16:
+            raise RuntimeError("LayerLauncher is the bf16 fast path")
+        dev = _require_gpu(k_cache, v_cache, global_end_index, local_end_index, freqs_table, q_like)
+        self.dev = dev
+        self.rows, self.tokens, self.heads = rows, tokens, heads
+        self.in_sig = (self._sig(q_like), self._sig(k_like), self._sig(v_like))
+        self.cache_sig = (k_cache.data_ptr(), v_cache.data_ptr(), tuple(k_cache.shape), tuple(k_cache.stride()),
+                          tuple(v_cache.stride()), global_end_index.data_ptr(), local_end_index.data_ptr())
+        self.k_cache, self.v_cache = k_cache, v_cache
+        self.lib = _capi.lib()
+        self.roped_q = torch.empty((rows, tokens, heads, HEAD_DIM), dtype=torch.bfloat16, device=dev)
+        self.sf = (C.c_int64 * rows)()
+        self.ds = (C.c_int64 * rows)()
+        self.ng = (C.c_int64 * rows)()
+        self.nl = (C.c_int64 * rows)()
+
+        ap = _capi.AppendParams()
+        ap.q_in_stride = _stride3(q_like, "q")
+        ap.k_in_stride = _stride3(k_like, "k")
+        ap.v_in_stride = _stride3(v_like, "v")
+        ap.q_out, ap.q_out_stride = self.roped_q.data_ptr(), _stride3(self.roped_q, "q_out")
+        ap.k_cache, ap.k_cache_stride = k_cache.data_ptr(), _stride3(k_cache, "k_cache")
+        ap.v_cache, ap.v_cache_stride = v_cache.data_ptr(), _stride3(v_cache, "v_cache")
+        ap.freqs, ap.freq_rows = freqs_table.data_ptr(), freqs_table.shape[0]
+        ap.dtype = _capi.DTYPE_BF16
+        ap.rows, ap.tokens, ap.heads, ap.head_dim = rows, tokens, heads, HEAD_DIM
+        ap.grid_f, ap.grid_h, ap.grid_w = (int(x) for x in grid)
+        ap.cache_tokens = k_cache.shape[1]
+        ap.start_frame = C.cast(self.sf, C.POINTER(C.c_int64))
+        ap.dst_start = C.cast(self.ds, C.POINTER(C.c_int64))
+        ap.global_end_index = global_end_index.data_ptr()
+        ap.local_end_index = local_end_index.data_ptr()
+        ap.new_global_end = C.cast(self.ng, C.POINTER(C.c_int64))
+        ap.new_local_end = C.cast(self.nl, C.POINTER(C.c_int64))
+        self.ap, self.ap_ref = ap, C.byref(ap)
+        self.freqs_table = freqs_table
+
+        at = _capi.AttnParams()
+        at.q, at.q_stride = self.roped_q.data_ptr(), _stride3(self.roped_q, "q")
+        at.k_cache, at.k_stride = k_cache.data_ptr(), _stride3(k_cache, "k_cache")
+        at.v_cache, at.v_stride = v_cache.data_ptr(), _stride3(v_cache, "v_cache")
+        at.rows, at.q_tokens, at.heads, at.head_dim = rows, tokens, heads, HEAD_DIM
+        self.at, self.at_ref = at, C.byref(at)
+        self.span = -1
+        self.out_stride = None
+        self.forced_splits = 0                       # 0 = the library's own choice
+
+    def matches(self, q, k, v, kv_cache, freqs_table) -> bool:
+        if (self._sig(q), self._sig(k), self._sig(v)) != self.in_sig or freqs_table is not self.freqs_table:
+            return False
+        kc, vc = kv_cache["k"], kv_cache["v"]
+        return self.cache_sig == (kc.data_ptr(), vc.data_ptr(), tuple(kc.shape), tuple(kc.stride()), tuple(vc.stride()),
+                                  kv_cache["global_end_index"].data_ptr(), kv_cache["local_end_index"].data_ptr())
+
+    def patch(self, q, k, v, start_frames, plan, seq_lens: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Fill in what changes from call to call and allocate the output
+        [rows, S, H, 128]; nothing is launched."""
+        ap, at = self.ap, self.at
+        for i in range(self.rows):
+            self.sf[i] = start_frames[i]
+            self.ds[i] = plan.dst_start[i]
+            self.ng[i] = plan.new_global_end[i]
+            self.nl[i] = plan.new_local_end[i]
+        ap.q_in, ap.k_in, ap.v_in = q.data_ptr(), k.data_ptr(), v.data_ptr()
+        stream = _stream_ptr(self.dev)
+        ap.stream = stream
+        span = plan.max_seq_len
+        if span != self.span:
+            self.span = span
+            at.max_seq_len = span
+            at.num_splits = self.forced_splits or self.lib.sdv2_swa_attn_default_splits(
+                self.rows, self.tokens, self.heads, span)
+            need = self.lib.sdv2_swa_attn_workspace_bytes(self.rows, self.tokens, self.heads, span, at.num_splits)
+            if need:
+                ws = _workspace(self.dev, need)
+                at.workspace, at.workspace_bytes = ws.data_ptr(), ws.numel()
+        elif at.workspace:
+            ws = _WORKSPACES[self.dev]              # may have been regrown by another shape
+            at.workspace, at.workspace_bytes = ws.data_ptr(), ws.numel()
+        out = torch.empty((self.rows, self.tokens, self.heads, HEAD_DIM), dtype=torch.bfloat16, device=self.dev)
+        if self.out_stride is None:
+            self.out_stride = _stride3(out, "out")
+            at.out_stride = self.out_stride
+        at.out = out.data_ptr()
+        at.seq_lens = seq_lens.data_ptr() if seq_lens is not None else None
+        at.stream = stream
+        return out
+
+    def run_append(self) -> None:
+        _capi.check(self.lib.sdv2_kv_append_rope(self.ap_ref), "sdv2_kv_append_rope")
+
+    def run_attention(self, stages: int = _capi.STAGE_ALL) -> None:
+        self.at.stages = stages
+        _capi.check(self.lib.sdv2_swa_attn_fwd(self.at_ref), "sdv2_swa_attn_fwd")
+
+    def launch(self, q, k, v, start_frames, plan, seq_lens: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Append + attention for one call; returns the attention output
+        [rows, S, H, 128].  The roped query stays in ``self.roped_q``."""
+        out = self.patch(q, k, v, start_frames, plan, seq_lens)
+        if _current_device_index() != self.dev.index:
+            with torch.cuda.device(self.dev):
+                self.run_append()
+                self.run_attention()
+        else:
+            self.run_append()
+            self.run_attention()
+        return out
 
 
 def flash_attn_with_kvcache(q, k_cache, v_cache, cache_seqlens=None):
