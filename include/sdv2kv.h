@@ -2,12 +2,13 @@
  * sdv2kv — C ABI of the MI355X (gfx950) ring-buffer KV-cache path for the
  * causal Wan DiT of StreamDiffusionV2.
  *
- * Two operators, both enqueued on a caller-supplied HIP stream, both working
- * on caller-owned device memory (the library owns nothing and, apart from the
- * lazily created constant RoPE state it is handed, keeps no mutable state):
+ * Three operators, all enqueued on a caller-supplied HIP stream, all working
+ * on caller-owned device memory (the library owns nothing and keeps no
+ * mutable state):
  *
- *   sdv2_kv_append_rope  fused RoPE-on-write chunk append
- *   sdv2_swa_attn_fwd    chunk-Q x (sink + window) K/V flash attention
+ *   sdv2_kv_append_rope   fused RoPE-on-write chunk append
+ *   sdv2_swa_attn_fwd     chunk-Q x (sink + window) K/V flash attention
+ *   sdv2_sink_similarity  adaptive sink refresh decision
  *
  * Tensors are addressed as [rows, tokens, heads, 128] with explicit element
  * strides for the first three dimensions; the last dimension is contiguous.
@@ -32,6 +33,7 @@ extern "C" {
 #define SDV2KV_ABI_VERSION 1
 #define SDV2_HEAD_DIM 128      /* causal_stream_inference.py:99-100 fixes 128 */
 #define SDV2_MAX_ROWS 16       /* rows (B) per sdv2_kv_append_rope call       */
+#define SDV2_MAX_SINK_FRAMES 16 /* sink frames per sdv2_sink_similarity call  */
 
 typedef enum sdv2_status {
   SDV2_OK = 0,
@@ -154,6 +156,48 @@ int sdv2_swa_attn_default_splits(int32_t rows, int32_t q_tokens, int32_t heads, 
 size_t sdv2_swa_attn_workspace_bytes(int32_t rows, int32_t q_tokens, int32_t heads,
                                      int32_t max_seq_len, int32_t num_splits);
 int sdv2_swa_attn_fwd(const sdv2_attn_params* p);
+
+/* ------------------------------------------------------------------------
+ * Adaptive sink refresh decision.
+ *
+ * Replaces models/wan/causal_model.py:284-299, which runs before the ring
+ * placement of a one-frame chunk when sink_size > 0 and adapt_sink_thr > -1:
+ *   k_sink_mean[j] = mean over tokens of cached K frame j   (j < sink_frames)
+ *   k_new_mean     = mean over tokens of rope(k_in)
+ *   sim[j] = (cos(k_sink_mean[j], k_new_mean) + cos(v_sink_mean[j], v_new_mean)) / 2
+ *   refresh = argmin_j sim[j] if min_j sim[j] < threshold else -1
+ * with the cosine taken over the flattened heads x 128 vector.  The caller
+ * reads `refresh` back and, for a row with refresh >= 0, puts
+ * (refresh + 1) * tokens at the head of that row's eviction queue (:297-299).
+ * k_in is the chunk's key BEFORE RoPE (the kernel rotates it exactly as
+ * sdv2_kv_append_rope does); the cache is read as it is before this call's
+ * append.  With bf16 tensors the means, both cosines and their sum are rounded
+ * to bf16, as the reference's bf16 tensors are.
+ * ---------------------------------------------------------------------- */
+typedef struct sdv2_sink_sim_params {
+  const void* k_in;            /* [B,S,H,128] new keys, not yet roped          */
+  const void* v_in;            /* [B,S,H,128] new values                       */
+  const void* k_cache;         /* [B,cap,H,128]                                */
+  const void* v_cache;
+  sdv2_stride3 k_in_stride, v_in_stride, k_cache_stride, v_cache_stride;
+  const double* freqs;         /* device, complex128 [freq_rows, 64] as (re,im) */
+  int32_t freq_rows;
+  int32_t dtype;               /* sdv2_dtype of the four tensors               */
+  int32_t rows, tokens, heads, head_dim;          /* B, S, H, 128              */
+  int32_t grid_h, grid_w;      /* tokens == grid_h * grid_w: exactly one frame */
+  int32_t sink_frames;         /* sink_size                                    */
+  float threshold;             /* adapt_sink_thr                               */
+  int64_t cache_tokens;        /* cap                                          */
+  const int64_t* start_frame;  /* host [B]: current_start // tokens            */
+  float* similarity;           /* device float [B, sink_frames]                */
+  int32_t* refresh;            /* device int32 [B]                             */
+  void* workspace;             /* device scratch for the frame means           */
+  size_t workspace_bytes;
+  void* stream;                /* hipStream_t                                  */
+} sdv2_sink_sim_params;
+
+size_t sdv2_sink_similarity_workspace_bytes(int32_t rows, int32_t heads, int32_t sink_frames);
+int sdv2_sink_similarity(const sdv2_sink_sim_params* p);
 
 /* ------------------------------------------------------------------------
  * Plain device-to-device copy of `bytes` bytes with the library's own 16-byte

@@ -220,6 +220,8 @@ class RingAttentionOracle:
         self.evict_idx: Optional[List[List[int]]] = None
         # what the last call did, for tests: per row (dst_start, dst_end)
         self.last_writes: List[Tuple[int, int]] = []
+        # per row the averaged similarities of the adaptive sink check, or None
+        self.last_sims: List[Optional[torch.Tensor]] = []
 
     def step(
         self,
@@ -251,6 +253,7 @@ class RingAttentionOracle:
 
         seq_lens: List[int] = []
         self.last_writes = []
+        self.last_sims = []
         for i, c_start in enumerate(starts):
             c_end = c_start + n_new
             queue = self.evict_idx[i]
@@ -268,6 +271,7 @@ class RingAttentionOracle:
                     frame_means(kv_cache["v"][i:i + 1, :sink_tokens], self.sink_size),
                     frame_means(v[i:i + 1], 1), dim=-1)
                 sim = (sim_k + sim_v) / 2
+                self.last_sims.append(sim.clone())
                 if sim.min() < self.adapt_sink_thr:
                     queue.insert(0, (int(torch.argmin(sim).item()) + 1) * frame_tokens)
 

@@ -35,6 +35,8 @@ EXPORTED_SYMBOLS = (
     "sdv2_swa_attn_default_splits",
     "sdv2_swa_attn_workspace_bytes",
     "sdv2_swa_attn_fwd",
+    "sdv2_sink_similarity_workspace_bytes",
+    "sdv2_sink_similarity",
     "sdv2_copy_bytes",
 )
 
@@ -81,6 +83,27 @@ class AttnParams(C.Structure):
     ]
 
 
+class SinkSimParams(C.Structure):
+    _fields_ = [
+        ("k_in", C.c_void_p), ("v_in", C.c_void_p), ("k_cache", C.c_void_p), ("v_cache", C.c_void_p),
+        ("k_in_stride", Stride3), ("v_in_stride", Stride3), ("k_cache_stride", Stride3), ("v_cache_stride", Stride3),
+        ("freqs", C.c_void_p),
+        ("freq_rows", C.c_int32),
+        ("dtype", C.c_int32),
+        ("rows", C.c_int32), ("tokens", C.c_int32), ("heads", C.c_int32), ("head_dim", C.c_int32),
+        ("grid_h", C.c_int32), ("grid_w", C.c_int32),
+        ("sink_frames", C.c_int32),
+        ("threshold", C.c_float),
+        ("cache_tokens", C.c_int64),
+        ("start_frame", C.POINTER(C.c_int64)),
+        ("similarity", C.c_void_p),
+        ("refresh", C.c_void_p),
+        ("workspace", C.c_void_p),
+        ("workspace_bytes", C.c_size_t),
+        ("stream", C.c_void_p),
+    ]
+
+
 _LIB: Optional[C.CDLL] = None
 
 
@@ -107,6 +130,10 @@ def lib() -> C.CDLL:
     handle.sdv2_swa_attn_workspace_bytes.argtypes = [C.c_int32] * 5
     handle.sdv2_swa_attn_fwd.restype = C.c_int
     handle.sdv2_swa_attn_fwd.argtypes = [C.POINTER(AttnParams)]
+    handle.sdv2_sink_similarity_workspace_bytes.restype = C.c_size_t
+    handle.sdv2_sink_similarity_workspace_bytes.argtypes = [C.c_int32] * 3
+    handle.sdv2_sink_similarity.restype = C.c_int
+    handle.sdv2_sink_similarity.argtypes = [C.POINTER(SinkSimParams)]
     handle.sdv2_copy_bytes.restype = C.c_int
     handle.sdv2_copy_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
     if handle.sdv2_abi_version() != ABI_VERSION:

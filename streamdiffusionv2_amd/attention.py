@@ -109,14 +109,24 @@ class RingKVPath:
         if len(self.evict_idx) < cache_rows:
             self.evict_idx = [list(self.evict_idx[0]) for _ in range(cache_rows)]
 
+        table = ops.device_freqs(freqs, q.device)
+        self.last_refresh = None
         if self.sink_size * frame_tokens > 0 and self.adapt_sink_thr > -1 and q.shape[1] <= frame_tokens:
-            raise NotImplementedError(
-                "adaptive sink refresh (causal_model.py:284-299) is not built yet; "
-                "set adapt_sink_thr = -1 for permanent sinks"
-            )
+            # adaptive sink refresh (causal_model.py:284-299): one fused
+            # reduction on the device, one small read-back for all rows
+            if q.shape[1] != frame_tokens:
+                raise RuntimeError(
+                    f"adaptive sink refresh needs one-frame chunks ({frame_tokens} tokens), got {q.shape[1]}"
+                )   # the reference's reshape(1, frame_seqlen, -1) fails the same way
+            _, refresh = ops.sink_similarity(
+                k, v, kv_cache["k"], kv_cache["v"], table, (h, w), [c // frame_tokens for c in starts],
+                self.sink_size, self.adapt_sink_thr)
+            self.last_refresh = refresh.tolist()
+            for i, frame in enumerate(self.last_refresh):
+                if frame >= 0:
+                    self.evict_idx[i].insert(0, (frame + 1) * frame_tokens)
 
         plan = ring.plan_append(kv_cache, self.evict_idx, starts, q.shape[1], frame_tokens, self.sink_size)
-        table = ops.device_freqs(freqs, q.device)
         span = plan.max_seq_len
         seq = None
         if any(n != span for n in plan.new_local_end):

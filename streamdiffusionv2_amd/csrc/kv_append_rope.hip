@@ -8,7 +8,7 @@
 // models/wan/causal_model.py:253-266, 321-322, 336-342.
 //
 // The kernel is a pure stream: 16-byte loads and stores, 16 lanes per
-// 256-byte head row, several heads per thread so the four table entries a
+// 256-byte head row, two heads per thread so the four table entries a
 // lane needs are fetched once and reused.  Algorithmic traffic per launch is
 // 6*B*S*H*128*sizeof(T) bytes (read q,k,v; write q', k', v).
 #include <hip/hip_runtime.h>
@@ -16,12 +16,13 @@
 
 #include "sdv2kv.h"
 #include "sdv2kv_internal.h"
+#include "rope_device.h"
 
 namespace {
 
 constexpr int kLanesPerRow = 16;            // 16 lanes x 8 elements = 128
 constexpr int kTokensPerBlock = 16;         // 256 threads
-constexpr int kHeadsPerThread = 4;
+constexpr int kHeadsPerThread = 2;        // measured best of 1 / 2 / 4 at every workload size
 
 struct AppendKernelArgs {
   const void* q_in;
@@ -42,70 +43,6 @@ struct AppendKernelArgs {
   int64_t new_global[SDV2_MAX_ROWS];
   int64_t new_local[SDV2_MAX_ROWS];
 };
-
-template <typename T>
-struct Vec8;
-
-template <>
-struct Vec8<uint16_t> {                     // bf16 bit patterns
-  uint4 raw;
-  __device__ static Vec8 load(const uint16_t* p) {
-    Vec8 v;
-    v.raw = *reinterpret_cast<const uint4*>(p);
-    return v;
-  }
-  __device__ void store(uint16_t* p) const { *reinterpret_cast<uint4*>(p) = raw; }
-  __device__ double get(int i) const {
-    const uint32_t w = (&raw.x)[i >> 1];
-    const uint32_t bits = (i & 1) ? (w & 0xffff0000u) : (w << 16);
-    return static_cast<double>(__uint_as_float(bits));
-  }
-  __device__ void set_pair(int p, double re, double im) {
-    (&raw.x)[p] = sdv2::f32_to_bf16_rne(static_cast<float>(re)) |
-                  (sdv2::f32_to_bf16_rne(static_cast<float>(im)) << 16);
-  }
-};
-
-template <>
-struct Vec8<float> {
-  float4 lo, hi;
-  __device__ static Vec8 load(const float* p) {
-    Vec8 v;
-    v.lo = *reinterpret_cast<const float4*>(p);
-    v.hi = *reinterpret_cast<const float4*>(p + 4);
-    return v;
-  }
-  __device__ void store(float* p) const {
-    *reinterpret_cast<float4*>(p) = lo;
-    *reinterpret_cast<float4*>(p + 4) = hi;
-  }
-  __device__ double get(int i) const {
-    return static_cast<double>(i < 4 ? (&lo.x)[i] : (&hi.x)[i - 4]);
-  }
-  __device__ void set_pair(int p, double re, double im) {
-    float* dst = p < 2 ? &lo.x + 2 * p : &hi.x + 2 * (p - 2);
-    dst[0] = static_cast<float>(re);
-    dst[1] = static_cast<float>(im);
-  }
-};
-
-// (a + bi)(c + di) with every product and sum rounded separately, as the
-// reference's complex128 multiply on the CPU does.
-template <typename T>
-__device__ __forceinline__ Vec8<T> rotate(const Vec8<T>& x, const double2 (&cs)[4]) {
-#pragma clang fp contract(off)
-  Vec8<T> y;
-#pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    const double a = x.get(2 * p), b = x.get(2 * p + 1);
-    const double ac = a * cs[p].x;
-    const double bd = b * cs[p].y;
-    const double ad = a * cs[p].y;
-    const double bc = b * cs[p].x;
-    y.set_pair(p, ac - bd, ad + bc);
-  }
-  return y;
-}
 
 template <typename T, bool kWithQ>
 __global__ __launch_bounds__(kLanesPerRow * kTokensPerBlock)
@@ -128,12 +65,7 @@ void kv_append_rope_kernel(const AppendKernelArgs a) {
   const int64_t frame = a.start_frame[row] + fi;
 
   double2 cs[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int p = lane * 4 + j;
-    const int64_t pos = p < a.split_t ? frame : (p < a.split_h ? hi : wi);
-    cs[j] = a.freqs[pos * a.pairs + p];
-  }
+  sdv2::load_rotation(a.freqs, a.pairs, a.split_t, a.split_h, lane, frame, hi, wi, cs);
 
   const int64_t e0 = lane * 8;
   const int64_t dst_tok = a.dst_start[row] + tok;
@@ -144,14 +76,14 @@ void kv_append_rope_kernel(const AppendKernelArgs a) {
   T* kc = static_cast<T*>(a.k_cache) + row * a.k_st.row + dst_tok * a.k_st.token + e0;
   T* vc = static_cast<T*>(a.v_cache) + row * a.v_st.row + dst_tok * a.v_st.token + e0;
 
-  Vec8<T> q[kHeadsPerThread], k[kHeadsPerThread], v[kHeadsPerThread];
+  sdv2::Vec8<T> q[kHeadsPerThread], k[kHeadsPerThread], v[kHeadsPerThread];
 #pragma unroll
   for (int j = 0; j < kHeadsPerThread; ++j) {
     const int h = head0 + j;
     if (h < a.heads) {
-      k[j] = Vec8<T>::load(ki + h * a.k_in_st.head);
-      v[j] = Vec8<T>::load(vi + h * a.v_in_st.head);
-      if (kWithQ) q[j] = Vec8<T>::load(qi + h * a.q_in_st.head);
+      k[j] = sdv2::Vec8<T>::load(ki + h * a.k_in_st.head);
+      v[j] = sdv2::Vec8<T>::load(vi + h * a.v_in_st.head);
+      if (kWithQ) q[j] = sdv2::Vec8<T>::load(qi + h * a.q_in_st.head);
     }
   }
 #pragma unroll
@@ -159,8 +91,8 @@ void kv_append_rope_kernel(const AppendKernelArgs a) {
     const int h = head0 + j;
     if (h < a.heads) {
       v[j].store(vc + h * a.v_st.head);
-      rotate(k[j], cs).store(kc + h * a.k_st.head);
-      if (kWithQ) rotate(q[j], cs).store(qo + h * a.q_out_st.head);
+      sdv2::rotate(k[j], cs).store(kc + h * a.k_st.head);
+      if (kWithQ) sdv2::rotate(q[j], cs).store(qo + h * a.q_out_st.head);
     }
   }
 }

@@ -228,6 +228,69 @@ def swa_attention(
     return out
 
 
+_SIM_WORKSPACES: dict = {}
+
+
+def sink_similarity(
+    k: torch.Tensor,
+    v: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    freqs_table: torch.Tensor,
+    grid_hw: Sequence[int],
+    start_frames: Sequence[int],
+    sink_frames: int,
+    threshold: float,
+):
+    """Adaptive sink refresh decision (causal_model.py:284-299) for a
+    one-frame chunk, before its append.
+
+    k is the chunk's key BEFORE RoPE, v its value, both [B,S,H,128]; the caches
+    are read as they are.  Returns (similarity float32 [B, sink_frames],
+    refresh int32 [B]) on the device: refresh[i] is the sink frame of row i to
+    overwrite next, or -1.
+    """
+    dev = _require_gpu(k, v, k_cache, v_cache, freqs_table)
+    if not (k.dtype == v.dtype == k_cache.dtype == v_cache.dtype):
+        raise RuntimeError("k, v and the caches must share one dtype")
+    rows, tokens, heads, _ = k.shape
+    if tuple(v.shape) != tuple(k.shape):
+        raise RuntimeError("k and v must have one shape")
+    if k_cache.shape[0] < rows or v_cache.shape != k_cache.shape or k_cache.shape[2] != heads:
+        raise RuntimeError(f"cache {tuple(k_cache.shape)} does not match the chunk {tuple(k.shape)}")
+    lib = _capi.lib()
+    need = lib.sdv2_sink_similarity_workspace_bytes(rows, heads, sink_frames)
+    ws = _SIM_WORKSPACES.get(dev)
+    if ws is None or ws.numel() < need:
+        ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+        _SIM_WORKSPACES[dev] = ws
+    similarity = torch.empty((rows, sink_frames), dtype=torch.float32, device=dev)
+    refresh = torch.empty((rows,), dtype=torch.int32, device=dev)
+
+    p = _capi.SinkSimParams()
+    p.k_in, p.k_in_stride = k.data_ptr(), _stride3(k, "k")
+    p.v_in, p.v_in_stride = v.data_ptr(), _stride3(v, "v")
+    p.k_cache, p.k_cache_stride = k_cache.data_ptr(), _stride3(k_cache, "k_cache")
+    p.v_cache, p.v_cache_stride = v_cache.data_ptr(), _stride3(v_cache, "v_cache")
+    p.freqs, p.freq_rows = freqs_table.data_ptr(), freqs_table.shape[0]
+    if k.dtype not in _DTYPES:
+        raise RuntimeError(f"unsupported dtype {k.dtype}")
+    p.dtype = _DTYPES[k.dtype]
+    p.rows, p.tokens, p.heads, p.head_dim = rows, tokens, heads, HEAD_DIM
+    p.grid_h, p.grid_w = int(grid_hw[0]), int(grid_hw[1])
+    p.sink_frames = int(sink_frames)
+    p.threshold = float(threshold)
+    p.cache_tokens = k_cache.shape[1]
+    starts = _i64_array(start_frames)
+    p.start_frame = C.cast(starts, C.POINTER(C.c_int64))
+    p.similarity, p.refresh = similarity.data_ptr(), refresh.data_ptr()
+    p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
+    p.stream = _stream_ptr(dev)
+    with torch.cuda.device(dev):
+        _capi.check(lib.sdv2_sink_similarity(C.byref(p)), "sdv2_sink_similarity")
+    return similarity, refresh
+
+
 class LayerLauncher:
     """Pre-built launch descriptors for one layer's (append, attention) pair.
 

@@ -1,0 +1,195 @@
+"""GPU parity of the adaptive sink refresh (causal_model.py:284-299) against
+the CPU oracle: the similarity operator on its own (both dtypes, both cache
+layouts) and whole streams with the refresh switched on, where every decision,
+every slot and the cache contents must be identical.
+
+The decision compares an averaged cosine similarity with a threshold.  Means
+are fp32 sums in a different order on the two sides and are then rounded to
+bf16, so similarities agree to about one bf16 step (tolerance 1e-2 for bf16,
+1e-5 for fp32).  The streams use inputs with a strong per-chunk direction so
+that every decision of the oracle has a margin of at least 0.03 to the
+threshold and to the runner-up frame (asserted), which makes the decisions
+comparable exactly.
+"""
+import pytest
+import torch
+
+from oracle import sdv2_oracle as oracle
+
+GRID = (1, 6, 8)
+FT = 48
+THR = 0.2
+MARGIN = 0.03
+
+
+def directed_chunk(gen, rows, heads, dtype, basis, scene=None, scale=0.25):
+    """q, k, v [rows, FT, heads, 128]: noise plus a chunk-wide direction from
+    the span of `basis` (the same on every token, so it survives the frame
+    mean; RoPE averages part of k's away).  With `scene` (coefficients [3]) the
+    direction stays near that scene's, so consecutive chunks look alike until
+    the scene changes."""
+    shape = (rows, FT, heads, 128)
+    q = torch.randn(shape, generator=gen) * scale
+    k = torch.randn(shape, generator=gen) * scale
+    v = torch.randn(shape, generator=gen) * scale
+    for r in range(rows):
+        cv = torch.randn(basis.shape[0], generator=gen)
+        ck = torch.randn(basis.shape[0], generator=gen)
+        if scene is not None:
+            cv, ck = 2 * scene + 0.3 * cv, 2 * scene + 0.3 * ck
+        v[r] += (cv @ basis).reshape(1, heads, 128)
+        k[r] += (ck @ basis).reshape(1, heads, 128)
+    return q.to(dtype), k.to(dtype), v.to(dtype)
+
+
+def oracle_margins_ok(sims):
+    """Every decision is clear of the threshold and has a clear minimum.
+    Frames never written give exactly 0 on both sides, so a tie at 0 is exact
+    and resolves to the first such frame everywhere."""
+    for s in sims:
+        s = s.float().sort().values
+        if abs(s[0].item() - THR) < MARGIN:
+            return False
+        tie_at_zero = s[0].item() == 0.0 and s[1].item() == 0.0
+        if s[0].item() < THR and not tie_at_zero and (s[1] - s[0]).item() < MARGIN:
+            return False
+    return True
+
+
+def test_stream_recipe_has_clear_margins_on_the_oracle():
+    """CPU check of the test data itself: the seeds used below give the oracle
+    clear decisions of both kinds (refresh and keep)."""
+    for dtype, seed, rows in ((torch.bfloat16, 10, 1), (torch.bfloat16, 36, 2)):
+        sims, refreshed = _oracle_stream(dtype, seed, rows, calls=12)[1:]
+        assert oracle_margins_ok(sims), [s.tolist() for s in sims]
+        assert 0 < refreshed < len(sims)
+
+
+def _oracle_stream(dtype, seed, rows, calls, heads=2, sink=3, cache_frames=6):
+    gen = torch.Generator().manual_seed(seed)
+    basis = torch.randn(3, heads * 128, generator=gen)
+    freqs = oracle.build_freqs()
+    cache = oracle.new_kv_cache(1, 1, cache_frames * FT, heads, 1, dtype=dtype)[0]
+    layer = oracle.RingAttentionOracle(sink_size=sink, adapt_sink_thr=THR)
+    record, sims, refreshed = [], [], 0
+    for call in range(calls):
+        if call == 1 and rows > 1:
+            oracle.replicate_for_stream_batch([cache], rows)
+        n = 1 if call == 0 else rows
+        starts = [max(call - r, 0) * FT for r in range(n)]
+        if call % 4 == 0:
+            scene = torch.randn(3, generator=gen)       # a scene cut every fourth chunk
+        q, k, v = directed_chunk(gen, n, heads, dtype, basis, scene)
+        out, roped_q, seq = layer.step(q, k, v, [GRID] * n, freqs, cache, starts)
+        sims.extend(layer.last_sims)
+        refreshed += sum(1 for s in layer.last_sims if s.min().item() < THR)
+        record.append(dict(q=q, k=k, v=v, starts=starts, out=out, roped_q=roped_q, seq=seq,
+                           writes=list(layer.last_writes), queue=[list(x) for x in layer.evict_idx],
+                           sims=[s.clone() for s in layer.last_sims],
+                           cache_k=cache["k"].clone(), cache_v=cache["v"].clone()))
+    return record, sims, refreshed
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, 1e-2), (torch.float32, 1e-5)])
+@pytest.mark.parametrize("head_major", [True, False])
+def test_similarity_operator(gpu_device, dtype, tol, head_major):
+    from streamdiffusionv2_amd import ops, rope
+
+    print(f"sink similarity operator: {dtype} head_major={head_major}", flush=True)
+    rows, heads, sink, cap = 2, 3, 3, 5 * FT
+    gen = torch.Generator().manual_seed(11)
+    basis = torch.randn(3, heads * 128, generator=gen)
+    freqs = rope.build_freqs()
+    _, k, v = directed_chunk(gen, rows, heads, dtype, basis)
+    ck = torch.cat([directed_chunk(gen, rows, heads, dtype, basis)[1] for _ in range(5)], dim=1)
+    cv = torch.cat([directed_chunk(gen, rows, heads, dtype, basis)[2] for _ in range(5)], dim=1)
+    start_frames = [7, 2]
+
+    roped = oracle.causal_rope_apply(k, [GRID] * rows, oracle.build_freqs(), start_frames).type_as(v)
+    want = []
+    for r in range(rows):
+        def means(t, frames):
+            return t.reshape(frames, FT, -1).mean(1)
+        sk = torch.cosine_similarity(means(ck[r:r + 1, :sink * FT], sink), means(roped[r:r + 1], 1), dim=-1)
+        sv = torch.cosine_similarity(means(cv[r:r + 1, :sink * FT], sink), means(v[r:r + 1], 1), dim=-1)
+        want.append(((sk + sv) / 2).float())
+    want = torch.stack(want)
+
+    def on_gpu(t):
+        if head_major:
+            return t.permute(0, 2, 1, 3).contiguous().to(gpu_device).permute(0, 2, 1, 3)
+        return t.to(gpu_device)
+
+    table = ops.device_freqs(freqs, gpu_device)
+    sim, refresh = ops.sink_similarity(k.to(gpu_device), v.to(gpu_device), on_gpu(ck), on_gpu(cv), table,
+                                       GRID[1:], start_frames, sink, THR)
+    torch.cuda.synchronize()
+    assert (sim.cpu() - want).abs().max().item() <= tol, (sim.cpu(), want)
+    for r in range(rows):
+        lo = want[r].min().item()
+        if abs(lo - THR) > MARGIN:
+            expect = int(want[r].argmin()) if lo < THR else -1
+            assert refresh[r].item() == expect
+    # an impossible threshold never refreshes, a generous one picks the minimum
+    _, never = ops.sink_similarity(k.to(gpu_device), v.to(gpu_device), on_gpu(ck), on_gpu(cv), table,
+                                   GRID[1:], start_frames, sink, -0.999)
+    assert never.cpu().tolist() == [-1] * rows
+    sim2, always = ops.sink_similarity(k.to(gpu_device), v.to(gpu_device), on_gpu(ck), on_gpu(cv), table,
+                                       GRID[1:], start_frames, sink, 1.5)
+    assert always.cpu().tolist() == sim2.argmin(dim=1).cpu().tolist()
+
+
+@pytest.mark.gpu
+def test_similarity_operator_rejects_bad_calls(gpu_device):
+    from streamdiffusionv2_amd import ops, rope
+
+    table = ops.device_freqs(rope.build_freqs(), gpu_device)
+    x = torch.zeros(1, FT, 2, 128, dtype=torch.bfloat16, device=gpu_device)
+    cache = torch.zeros(1, 4 * FT, 2, 128, dtype=torch.bfloat16, device=gpu_device)
+    two_frames = torch.zeros(1, 2 * FT, 2, 128, dtype=torch.bfloat16, device=gpu_device)
+    with pytest.raises(RuntimeError):       # more than one frame
+        ops.sink_similarity(two_frames, two_frames, cache, cache, table, GRID[1:], [0], 2, THR)
+    with pytest.raises(RuntimeError):       # sink larger than the cache
+        ops.sink_similarity(x, x, cache, cache, table, GRID[1:], [0], 5, THR)
+    with pytest.raises(RuntimeError):       # frame beyond the RoPE table
+        ops.sink_similarity(x, x, cache, cache, table, GRID[1:], [1024], 2, THR)
+    with pytest.raises(RuntimeError):       # CPU tensors: no fallback
+        ops.sink_similarity(x.cpu(), x.cpu(), cache.cpu(), cache.cpu(), table, GRID[1:], [0], 2, THR)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed,rows", [(10, 1), (36, 2)])
+def test_stream_with_refresh(gpu_device, seed, rows):
+    from streamdiffusionv2_amd import ring, rope
+    from streamdiffusionv2_amd.attention import RingKVPath
+
+    print(f"adaptive sink stream: seed={seed} rows={rows}", flush=True)
+    heads, sink, cache_frames, calls = 2, 3, 6, 12
+    record, sims, refreshed = _oracle_stream(torch.bfloat16, seed, rows, calls)
+    assert oracle_margins_ok(sims) and 0 < refreshed < len(sims)
+
+    freqs = rope.build_freqs()
+    cache = ring.new_kv_cache(1, 1, cache_frames * FT, heads, 1, device=gpu_device)[0]
+    path = RingKVPath(sink_size=sink, adapt_sink_thr=THR)
+    for call, rec in enumerate(record):
+        if call == 1 and rows > 1:
+            ring.replicate_for_stream_batch([cache], rows)
+        n = len(rec["starts"])
+        got, got_q = path.attend(rec["q"].to(gpu_device), rec["k"].to(gpu_device), rec["v"].to(gpu_device),
+                                 torch.tensor([GRID] * n), freqs, cache, rec["starts"], return_roped_query=True)
+        torch.cuda.synchronize()
+        want_refresh = [int(s.argmin()) if s.min().item() < THR else -1 for s in rec["sims"]]
+        assert path.last_refresh == want_refresh, call
+        assert path.evict_idx == rec["queue"], call
+        assert path.last_plan.new_local_end == rec["seq"], call
+        assert [(a, a + FT) for a in path.last_plan.dst_start] == rec["writes"], call
+        assert torch.equal(got_q.cpu().view(torch.int16), rec["roped_q"].view(torch.int16)), call
+        for name in ("k", "v"):
+            assert torch.equal(cache[name].cpu().view(torch.int16), rec["cache_" + name].view(torch.int16)), (call, name)
+        # the directed values reach several units, so the unit-scale bounds
+        # (max-abs 2e-2, mean-abs 2e-3) are taken relative to the largest output
+        want = oracle.attention_fp32_reference(rec["roped_q"], rec["cache_k"], rec["cache_v"], rec["seq"])
+        unit = max(1.0, want.abs().max().item())
+        err = (got.float().cpu() - want).abs()
+        assert err.max().item() <= 2e-2 * unit and err.mean().item() <= 2e-3 * unit, call
