@@ -49,6 +49,8 @@ def parse_args():
     ap.add_argument("--cpu-layers", type=int, default=2)
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="only run the library's plain copy kernel on MIB mebibytes (counter calibration)")
+    ap.add_argument("--skip-mfma-reference", action="store_true",
+                    help="do not time the vendor bf16 GEMM that shows what this box sustains on MFMA")
     return ap.parse_args()
 
 
@@ -164,6 +166,34 @@ def gpu_bench(args, w):
         "merge_ms": t_merge,
         "splits": splits,
     }
+
+
+def mfma_reference(n=8192, iters=20):
+    """What the box sustains on dense bf16 MFMA work: the vendor GEMM behind
+    torch.matmul (hipBLASLt / rocBLAS) on n^3 problems, with random operands
+    (the realistic case: the chip's clock under MFMA load depends on how much
+    the data toggles) and with all-zero operands (the quietest case).  Context
+    for the attention kernel's roofline fraction, not part of the timed path."""
+    dev = torch.device("cuda:0")
+    out = {"n": n, "unit": "TFLOP/s", "source": "torch.matmul bf16 (vendor GEMM)"}
+    for kind in ("random", "zeros"):
+        if kind == "random":
+            a = torch.randn(n, n, device=dev).bfloat16()
+            b = torch.randn(n, n, device=dev).bfloat16()
+        else:
+            a = torch.zeros(n, n, device=dev, dtype=torch.bfloat16)
+            b = torch.zeros(n, n, device=dev, dtype=torch.bfloat16)
+        for _ in range(3):
+            a @ b
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            a @ b
+        e1.record()
+        torch.cuda.synchronize()
+        out[kind] = 2 * n ** 3 / (e0.elapsed_time(e1) / iters) / 1e9
+    return out
 
 
 def cpu_baseline(args, w):
@@ -294,6 +324,10 @@ def main():
         },
         "kernel_ms_per_layer": {"append": g["append_ms"], "attn": g["attn_ms"], "merge": g["merge_ms"]},
     }
+    if not args.skip_mfma_reference:
+        ref = mfma_reference()
+        ref["attention_vs_random"] = achieved_tflops / ref["random"]
+        result["mfma_reference"] = ref
     if not args.skip_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(args, w)
     print(json.dumps(result))

@@ -316,6 +316,38 @@ class RingAttentionOracle:
         return out, roped_q, seq_lens
 
 
+def new_crossattn_cache(num_layers: int, batch_size: int, heads: int, dtype=torch.bfloat16,
+                        text_tokens: int = 512) -> List[dict]:
+    """causal_stream_inference.py:109-122."""
+    return [
+        {
+            "k": torch.zeros(batch_size, text_tokens, heads, 128, dtype=dtype),
+            "v": torch.zeros(batch_size, text_tokens, heads, 128, dtype=dtype),
+            "is_init": False,
+        }
+        for _ in range(num_layers)
+    ]
+
+
+def cross_attention_with_cache(q: torch.Tensor, make_kv, context_lens, crossattn_cache: Optional[dict]):
+    """The cache logic of WanT2VCrossAttention.forward
+    (wan_base/modules/model.py:172-192) around the attention operator:
+    ``make_kv()`` stands for the K/V projections of the text context and is
+    only called when the cache is absent or not initialised; an initialised
+    cache is read as it is.  Attention = softmax(q k^T / sqrt(128)) v over the
+    first context_lens[i] keys of row i (all keys when None)."""
+    if crossattn_cache is not None and crossattn_cache["is_init"]:
+        k, v = crossattn_cache["k"], crossattn_cache["v"]
+    else:
+        k, v = make_kv()
+        if crossattn_cache is not None:
+            crossattn_cache["is_init"] = True
+            crossattn_cache["k"] = k
+            crossattn_cache["v"] = v
+    lens = [k.shape[1]] * q.shape[0] if context_lens is None else [int(n) for n in context_lens]
+    return attention_with_kvcache(q, k, v, torch.tensor(lens, dtype=torch.int32))
+
+
 # --------------------------------------------------------------------------
 # drivers: stream-batch shift register and chunk arithmetic
 # --------------------------------------------------------------------------

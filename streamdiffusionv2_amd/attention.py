@@ -217,3 +217,44 @@ class CausalWanSelfAttention(nn.Module, RingKVPath):
         v = self.v(x).view(b, s, n, d)
         out = self.attend(q, k, v, grid_sizes, freqs, kv_cache, current_start)
         return self.o(out.flatten(2))
+
+
+class WanT2VCrossAttention(nn.Module):
+    """Text cross-attention with the per-prompt K/V cache
+    (wan_base/modules/model.py:160-196): same constructor, child module names
+    and ``forward(x, context, context_lens, crossattn_cache=None)``.  The first
+    call of a prompt projects the context and stores K/V in the cache dict;
+    later calls read them.  The attention itself is the library's kernel on
+    the 512 cached keys."""
+
+    def __init__(self, dim, num_heads, window_size=(-1, -1), qk_norm=True, eps=1e-6):
+        assert dim % num_heads == 0
+        super().__init__()
+        self.dim = dim
+        self.num_heads = num_heads
+        self.head_dim = dim // num_heads
+        self.window_size = window_size
+        self.qk_norm = qk_norm
+        self.eps = eps
+        self.q = nn.Linear(dim, dim)
+        self.k = nn.Linear(dim, dim)
+        self.v = nn.Linear(dim, dim)
+        self.o = nn.Linear(dim, dim)
+        self.norm_q = WanRMSNorm(dim, eps=eps) if qk_norm else nn.Identity()
+        self.norm_k = WanRMSNorm(dim, eps=eps) if qk_norm else nn.Identity()
+
+    def forward(self, x, context, context_lens, crossattn_cache=None):
+        """x [B, L1, dim]; context [B, L2, dim]; context_lens [B] or None."""
+        b, n, d = x.size(0), self.num_heads, self.head_dim
+        q = self.norm_q(self.q(x)).view(b, -1, n, d)
+        if crossattn_cache is not None and crossattn_cache["is_init"]:
+            k, v = crossattn_cache["k"], crossattn_cache["v"]
+        else:
+            k = self.norm_k(self.k(context)).view(b, -1, n, d)
+            v = self.v(context).view(b, -1, n, d)
+            if crossattn_cache is not None:
+                crossattn_cache["is_init"] = True
+                crossattn_cache["k"] = k
+                crossattn_cache["v"] = v
+        out = ops.flash_attention(q, k, v, k_lens=context_lens)
+        return self.o(out.flatten(2))

@@ -431,6 +431,35 @@ def flash_attn_with_kvcache(q, k_cache, v_cache, cache_seqlens=None):
     return swa_attention(q, k_cache, v_cache, cache_seqlens)
 
 
+def flash_attention(q, k, v, q_lens=None, k_lens=None, dropout_p=0.0, softmax_scale=None, q_scale=None,
+                    causal=False, window_size=(-1, -1), deterministic=False, dtype=torch.bfloat16, version=None):
+    """The reference's generic attention entry (wan_base/modules/attention.py,
+    ``flash_attention``) for the cases the cached inference path uses:
+    cross-attention of a chunk against the cached text keys / values
+    (wan_base/modules/model.py:192), i.e. no causal mask, no window, no dropout,
+    every query row valid.  k / v may be ``expand``-ed views (row stride 0, as
+    causal_stream_inference.py:227-228 makes them).  Inputs that are not bf16
+    are computed in bf16 and the result is returned in q's dtype, as the
+    reference does with its ``dtype`` argument."""
+    if causal or tuple(window_size) != (-1, -1) or dropout_p or q_lens is not None:
+        raise NotImplementedError("flash_attention here covers the cached inference path: "
+                                  "causal=False, window_size=(-1, -1), dropout_p=0, q_lens=None")
+    if dtype != torch.bfloat16:
+        raise NotImplementedError("the attention kernel computes in bf16")
+    out_dtype = q.dtype
+    scale = None
+    if q_scale is not None or softmax_scale is not None:
+        scale = (q_scale if q_scale is not None else 1.0) * \
+                (softmax_scale if softmax_scale is not None else HEAD_DIM ** -0.5)
+    if k_lens is not None:
+        k_lens = k_lens.to(device=q.device, dtype=torch.int32).contiguous()
+    qb, kb, vb = (t if t.dtype == torch.bfloat16 else t.to(torch.bfloat16) for t in (q, k, v))
+    if qb.stride(-1) != 1:
+        qb = qb.contiguous()
+    out = swa_attention(qb, kb, vb, k_lens, softmax_scale=scale)
+    return out if out_dtype == torch.bfloat16 else out.to(out_dtype)
+
+
 def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
     """Plain 16-byte-vector copy with the library's own kernel (used to scale
     hardware counters against a transfer of known size)."""

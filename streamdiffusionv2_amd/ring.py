@@ -76,6 +76,29 @@ def replicate_for_stream_batch(kv_cache: List[dict], batch_size: int) -> None:
         entry.pop(_MIRROR_KEY, None)
 
 
+def new_crossattn_cache(num_layers: int, batch_size: int, heads: int, dtype=torch.bfloat16, device="cuda",
+                        text_tokens: int = 512) -> List[dict]:
+    """Per-layer cross-attention cache (causal_stream_inference.py:109-122):
+    ``k`` / ``v`` zeros [B, 512, H, 128] and ``is_init`` False; the first
+    cross-attention call of a prompt fills it (wan_base/modules/model.py:174-184)."""
+    return [
+        {
+            "k": torch.zeros(batch_size, text_tokens, heads, 128, dtype=dtype, device=device),
+            "v": torch.zeros(batch_size, text_tokens, heads, 128, dtype=dtype, device=device),
+            "is_init": False,
+        }
+        for _ in range(num_layers)
+    ]
+
+
+def expand_crossattn_for_stream_batch(crossattn_cache: List[dict], batch_size: int) -> None:
+    """Stream-batch expansion of the text cache (causal_stream_inference.py:227-228):
+    a broadcast view, every row reads the same 512 keys (row stride 0)."""
+    for entry in crossattn_cache:
+        entry["k"] = entry["k"].expand(batch_size, -1, -1, -1)
+        entry["v"] = entry["v"].expand(batch_size, -1, -1, -1)
+
+
 @dataclass
 class _IndexMirror:
     g_tensor: torch.Tensor
