@@ -118,6 +118,8 @@ class KVStreamPipeline:
         self.kv_cache_starts: Optional[List[int]] = None
         self.kv_cache_ends: Optional[List[int]] = None
         self.batch_size = 1
+        self.active_mode = "batch"
+        self._batch_state_refs: Optional[dict] = None
         self._cache_factory = cache_factory or ring.new_kv_cache
         self._replicate = ring.replicate_for_stream_batch
 
@@ -172,6 +174,55 @@ class KVStreamPipeline:
         for _ in self.denoising_step_list:
             out = self.generator(noise, self.kv_cache1, [current_start])
         return out
+
+
+    # -- demo/vid2vid.py:113-135 -------------------------------------------
+    _CACHE_TENSORS = ("k", "v", "global_end_index", "local_end_index")
+
+    def enter_wo_batch(self) -> None:
+        """Switch a running stream batch to sequential (no-batch) denoising:
+        every cache dict is narrowed to views of its row 0, the batch tensors
+        are kept aside untouched.  Nothing is copied."""
+        if self.active_mode == "wo_batch":
+            return
+        self._batch_state_refs = {
+            "kv_cache1": [{name: entry[name] for name in self._CACHE_TENSORS} for entry in self.kv_cache1],
+            "hidden_states": self.hidden_states,
+            "kv_cache_starts": self.kv_cache_starts,
+            "kv_cache_ends": self.kv_cache_ends,
+        }
+        for entry, saved in zip(self.kv_cache1, self._batch_state_refs["kv_cache1"]):
+            for name in self._CACHE_TENSORS:
+                entry[name] = saved[name][:1]
+        self.active_mode = "wo_batch"
+
+    # -- demo/vid2vid.py:137-198 -------------------------------------------
+    def return_to_batch(self, current_start: int, current_end: int) -> None:
+        """Back to the stream batch: row 0 (the only row the sequential mode
+        advanced) is copied over every other row of the batch tensors, each
+        row's eviction queue becomes a copy of row 0's, the pass counter is
+        rewound, the pipeline registers restart from the session position."""
+        if self.active_mode == "batch":
+            return
+        if self._batch_state_refs is None:
+            raise RuntimeError("Cannot restore batch mode before batch state has been captured")
+        for entry, saved in zip(self.kv_cache1, self._batch_state_refs["kv_cache1"]):
+            for name in self._CACHE_TENSORS:
+                t = saved[name]
+                if t.shape[0] > 1 and t.stride(0) != 0:
+                    t[1:].copy_(t[:1].expand_as(t[1:]))
+                entry[name] = t
+            if "total_steps" in entry:
+                entry["current_step"] = entry["total_steps"]
+        self.hidden_states = torch.zeros_like(self._batch_state_refs["hidden_states"])
+        n = len(self._batch_state_refs["kv_cache_starts"])
+        self.kv_cache_starts = [int(current_start)] * n
+        self.kv_cache_ends = [int(current_end)] * n
+        for path in self.generator.paths:
+            if isinstance(path.evict_idx, list) and path.evict_idx:
+                path.evict_idx = [list(path.evict_idx[0]) for _ in range(self.hidden_states.shape[0])]
+        self.active_mode = "batch"
+        self._batch_state_refs = None
 
 
 @dataclass

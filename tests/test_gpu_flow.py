@@ -11,40 +11,7 @@ from oracle import sdv2_oracle as oracle
 pytestmark = pytest.mark.gpu
 
 
-class OraclePath:
-    """Adapter: the oracle layer behind the attend() call of the package."""
-
-    def __init__(self):
-        self.inner = oracle.RingAttentionOracle()
-        self.trace = []
-
-    sink_size = property(lambda s: s.inner.sink_size, lambda s, v: setattr(s.inner, "sink_size", v))
-    adapt_sink_thr = property(lambda s: s.inner.adapt_sink_thr, lambda s, v: setattr(s.inner, "adapt_sink_thr", v))
-    evict_idx = property(lambda s: s.inner.evict_idx)
-
-    def attend(self, q, k, v, grid_sizes, freqs, kv_cache, current_start):
-        out, _, seq = self.inner.step(q, k, v, grid_sizes.tolist(), freqs, kv_cache, current_start)
-        self.trace.append((list(current_start), list(self.inner.last_writes), seq))
-        return out
-
-
-class TracedGpuPath:
-    def __init__(self):
-        from streamdiffusionv2_amd.attention import RingKVPath
-
-        self.inner = RingKVPath()
-        self.trace = []
-
-    sink_size = property(lambda s: s.inner.sink_size, lambda s, v: setattr(s.inner, "sink_size", v))
-    adapt_sink_thr = property(lambda s: s.inner.adapt_sink_thr, lambda s, v: setattr(s.inner, "adapt_sink_thr", v))
-    evict_idx = property(lambda s: s.inner.evict_idx)
-
-    def attend(self, q, k, v, grid_sizes, freqs, kv_cache, current_start):
-        out = self.inner.attend(q, k, v, grid_sizes, freqs, kv_cache, current_start)
-        plan = self.inner.last_plan
-        S = q.shape[1]
-        self.trace.append((list(current_start), [(d, d + S) for d in plan.dst_start], list(plan.new_local_end)))
-        return out
+from flow_helpers import OraclePath, TracedGpuPath  # noqa: E402
 
 
 @pytest.mark.parametrize("mode", ["single", "single-wo"])
@@ -106,3 +73,67 @@ def test_staged_flow_matches_oracle_flow(gpu_device, mode):
         assert gc["current_step"] == oc["current_step"]
     # the clamp was reached: last calls sit at the cache's last frame
     assert g_gen.paths[0].trace[-1][0][0] == g_pipe.kv_cache_length - g_pipe.frame_seq_length
+
+
+def test_switch_to_sequential_mode_and_back(gpu_device):
+    """Stream batch -> sequential (row-0 views) -> stream batch again
+    (demo/vid2vid.py:113-198) on the GPU path against the same driver with the
+    oracle plugged in: identical positions, slots, lengths, queues, indices
+    and pass counters after every call; close outputs."""
+    from streamdiffusionv2_amd import stream
+
+    H, W = 64, 96
+    layers, heads, fsl = 2, 2, 24
+
+    def build(device, factory, cache_factory=None):
+        gen = stream.SyntheticGenerator(layers, heads, device, seed=13, path_factory=factory,
+                                        sink_size=1, adapt_sink_thr=-1)
+        pipe = stream.KVStreamPipeline(gen, height=H, width=W, num_kv_cache=4, num_sink_tokens=1,
+                                       denoising_step_list=(700, 500, 0), cache_factory=cache_factory)
+        return gen, pipe
+
+    def cpu_cache_factory(n, b, cap, h, steps, dtype, device):
+        return oracle.new_kv_cache(n, b, cap, h, steps, dtype=dtype, device="cpu")
+
+    g_gen, g_pipe = build(gpu_device, TracedGpuPath)
+    o_gen, o_pipe = build("cpu", OraclePath, cpu_cache_factory)
+    o_pipe._replicate = oracle.replicate_for_stream_batch
+
+    gen = torch.Generator().manual_seed(9)
+    noises = [torch.randn(1, 1, 16, H // 8, W // 8, generator=gen).bfloat16() for _ in range(12)]
+    results = []
+    for pipe in (g_pipe, o_pipe):
+        dev = pipe.device
+        outs, pos = [], 0
+        outs.append(pipe.prepare(noises[0].to(dev), 0, fsl))
+        pos = fsl
+        for i in range(1, 4):
+            outs.append(pipe.inference_stream(noises[i].to(dev), pos, pos + fsl))
+            pos += fsl
+        pipe.enter_wo_batch()
+        assert pipe.active_mode == "wo_batch" and pipe.kv_cache1[0]["k"].shape[0] == 1
+        for i in range(4, 8):
+            outs.append(pipe.inference_wo_batch(noises[i].to(dev), pos, pos + fsl))
+            pos += fsl
+        pipe.return_to_batch(pos, pos + fsl)
+        assert pipe.active_mode == "batch" and pipe.kv_cache1[0]["k"].shape[0] == pipe.batch_size
+        for entry in pipe.kv_cache1:                      # row 0 was broadcast over the batch
+            for name in ("k", "v", "global_end_index", "local_end_index"):
+                assert all(torch.equal(entry[name][r], entry[name][0]) for r in range(1, pipe.batch_size))
+            assert entry["current_step"] == entry["total_steps"]
+        for i in range(8, 12):
+            outs.append(pipe.inference_stream(noises[i].to(dev), pos, pos + fsl))
+            pos += fsl
+        results.append(outs)
+    torch.cuda.synchronize()
+
+    for gp, op in zip(g_gen.paths, o_gen.paths):
+        assert gp.trace == op.trace
+        assert gp.evict_idx == op.evict_idx
+    for gc, oc in zip(g_pipe.kv_cache1, o_pipe.kv_cache1):
+        assert gc["global_end_index"].cpu().tolist() == oc["global_end_index"].tolist()
+        assert gc["local_end_index"].cpu().tolist() == oc["local_end_index"].tolist()
+        assert gc["current_step"] == oc["current_step"]
+    for g, o in zip(*results):
+        diff = (g.float().cpu() - o.float()).abs()
+        assert diff.max().item() < 0.15 and diff.mean().item() < 0.02
