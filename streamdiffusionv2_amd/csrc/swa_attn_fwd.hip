@@ -51,6 +51,7 @@ typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 typedef __attribute__((address_space(3))) char lds_char;
@@ -609,10 +610,11 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   // Every tile runs the same code and the loop body is three whole tiles with
   // a single way in and out, so the accumulators keep their registers from trip
   // to trip (the compiler must never be given a reason to move them while asm
-  // MFMAs are in flight).  The tile count is padded to a multiple of three:
-  // padding tiles, like the tail of a partial tile, have all their scores
-  // masked to -inf, so their weights are exact zeros against whatever finite
-  // data the buffers still hold.  In the first slot P(-1) is zero likewise.
+  // MFMAs are in flight).  Scores of keys at or beyond the end of the range (the
+  // tail of a partial tile, the look-ahead block of a tile that does not
+  // exist) are masked to -inf, so their weights are exact zeros against
+  // whatever finite data the buffers still hold.  In the first slot P(-1) is
+  // zero likewise.
   const int key_end = seq < tile_end * kKTile ? seq : tile_end * kKTile;
   auto row_sums_unsafe = [&]() {
     bool bad = false;
@@ -635,7 +637,7 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
     if (T + 3 < n) issue_k(T + 3, kB);
     if (T + 2 < n) issue_v(T + 2, kBPrev);
     slot<1, kLdsK(kBNext), kLdsVRel(kB), true, true, true>(c, qf, s, p, oacc, l_run, key0 + 32, key_end);
-    if (T < n) unsafe |= row_sums_unsafe();
+    unsafe |= row_sums_unsafe();
   };
   using B0 = std::integral_constant<int, 0>;
   using B1 = std::integral_constant<int, 1>;
@@ -646,13 +648,28 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
     __syncthreads();        // the first tiles and the Q fragments have arrived
     // S(0) alone fills the pipeline
     slot<1, kLdsK(0), 0, true, false, false>(c, qf, s, p, oacc, l_run, 0, key_end);
+    // Three tiles per trip, one per buffer; the last trip stops after the last
+    // real tile.  The skipped tiles sit behind uniform branches that no value
+    // is changed on, so the accumulators stay where they are on either way.
     for (int T = 0; T < n; T += 3) {
       do_tile(B0{}, T);
-      do_tile(B1{}, T + 1);
-      do_tile(B2{}, T + 2);
+      if (T + 1 < n) {
+        do_tile(B1{}, T + 1);
+        if (T + 2 < n) do_tile(B2{}, T + 2);
+      }
     }
-    // PV of the last block (odd -> p[1], second half of the tile in V buffer 2) empties the pipeline
-    slot<0, 0, kLdsVRel(2) + 32 * 256, false, true, false>(c, qf, s, p, oacc, l_run, 0, key_end);
+    // PV of the last block (odd -> p[1], second half of the last tile's V
+    // buffer) empties the pipeline.  The code addresses V buffer 2; the lane
+    // addresses are moved when the last tile sits in another buffer.
+    {
+      LaneConst cf = c;
+      const uint32_t shift = (uint32_t)(((n - 1) % kStages - 2) * kTileBytes);
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) cf.v_addr[db][j] = c.v_addr[db][j] + shift;
+      slot<0, 0, kLdsVRel(2) + 32 * 256, false, true, false>(cf, qf, s, p, oacc, l_run, 0, key_end);
+    }
     mfma_drain<0>(oacc, s);
 
     // Did any wave of the workgroup see an unsafe row sum?  (LDS is free now.)
@@ -668,38 +685,67 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   }
 
   // ---- epilogue ---------------------------------------------------------------
+  // A lane holds one query row's values scattered over the 128 dims, so direct
+  // stores would touch 32 rows with 16 or 32 bytes each.  Instead every wave
+  // stages one 32-row block at a time in its own 16 KB of the (now idle) LDS,
+  // 16-byte chunks XOR-swizzled by row, and writes whole rows: 256 bytes of bf16
+  // for the result of an unsplit call, 512 bytes of fp32 for the normalised
+  // partial result of a split call (plus its log-sum-exp).  LDS operations of
+  // one wave complete in order, so the block needs no barrier of its own.
+  __syncthreads();                    // every wave is done with the K / V buffers
+  lds_char* stage = lds + wave * 16384;
+  const int q0 = qtile * kQTile + wave * kQRowsPerWave;
 #pragma unroll
   for (int qb = 0; qb < kQB; ++qb) {
     const float l_tot = half_sum(l_run[qb]);
     const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-    if (q_row[qb] >= a.q_tokens) continue;
+    const int r = lane & 31;
     if (a.num_splits == 1) {
-      uint16_t* op = a.out + row * a.o_st.row + (int64_t)q_row[qb] * a.o_st.token + head * a.o_st.head;
 #pragma unroll
       for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          uint2 w;
-          w.x = pack_bf16x2(oacc[qb][db][4 * g] * inv, oacc[qb][db][4 * g + 1] * inv);
-          w.y = pack_bf16x2(oacc[qb][db][4 * g + 2] * inv, oacc[qb][db][4 * g + 3] * inv);
-          *reinterpret_cast<uint2*>(op + db * 32 + 8 * g + 4 * hf) = w;
+          u32x2 w;
+          w[0] = pack_bf16x2(oacc[qb][db][4 * g] * inv, oacc[qb][db][4 * g + 1] * inv);
+          w[1] = pack_bf16x2(oacc[qb][db][4 * g + 2] * inv, oacc[qb][db][4 * g + 3] * inv);
+          const int chunk = db * 4 + g;
+          *reinterpret_cast<__attribute__((address_space(3))) u32x2*>(
+              stage + r * 256 + ((chunk ^ (r & 15)) << 4) + hf * 8) = w;
         }
+      uint16_t* dst = a.out + row * a.o_st.row + head * a.o_st.head + (int64_t)(q0 + qb * 32) * a.o_st.token;
+      const int j = lane & 15;
+#pragma unroll
+      for (int it = 0; it < 8; ++it) {
+        const int rr = 4 * it + (lane >> 4);
+        const u32x4 w = *reinterpret_cast<__attribute__((address_space(3))) const u32x4*>(
+            stage + rr * 256 + ((j ^ (rr & 15)) << 4));
+        if (q0 + qb * 32 + rr < a.q_tokens) *reinterpret_cast<u32x4*>(dst + rr * a.o_st.token + j * 8) = w;
+      }
     } else {
-      const int64_t prow = (((int64_t)split * a.rows + row) * a.heads + head) * a.q_tokens + q_row[qb];
-      float* po = a.part_o + prow * kD;
 #pragma unroll
       for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          float4 w;
-          w.x = oacc[qb][db][4 * g] * inv;
-          w.y = oacc[qb][db][4 * g + 1] * inv;
-          w.z = oacc[qb][db][4 * g + 2] * inv;
-          w.w = oacc[qb][db][4 * g + 3] * inv;
-          *reinterpret_cast<float4*>(po + db * 32 + 8 * g + 4 * hf) = w;
+          f32x4 w;
+          w[0] = oacc[qb][db][4 * g] * inv;
+          w[1] = oacc[qb][db][4 * g + 1] * inv;
+          w[2] = oacc[qb][db][4 * g + 2] * inv;
+          w[3] = oacc[qb][db][4 * g + 3] * inv;
+          const int chunk = db * 8 + 2 * g + hf;
+          *reinterpret_cast<__attribute__((address_space(3))) f32x4*>(stage + r * 512 + ((chunk ^ r) << 4)) = w;
         }
-      if (hf == 0)
-        a.part_lse[prow] = l_tot > 0.f ? m_run[qb] * c.c2 + __builtin_amdgcn_logf(l_tot) : -INFINITY;
+      const int64_t prow0 = (((int64_t)split * a.rows + row) * a.heads + head) * a.q_tokens + q0 + qb * 32;
+      if (hf == 0 && q_row[qb] < a.q_tokens)
+        a.part_lse[prow0 + r] = l_tot > 0.f ? m_run[qb] * c.c2 + __builtin_amdgcn_logf(l_tot) : -INFINITY;
+      float* dst = a.part_o + prow0 * kD;
+      const int j = lane & 31;
+#pragma unroll
+      for (int it = 0; it < 16; ++it) {
+        const int rr = 2 * it + (lane >> 5);
+        const f32x4 w = *reinterpret_cast<__attribute__((address_space(3))) const f32x4*>(
+            stage + rr * 512 + ((j ^ rr) << 4));
+        if (q0 + qb * 32 + rr < a.q_tokens) *reinterpret_cast<f32x4*>(dst + rr * kD + j * 4) = w;
+      }
     }
   }
 }
