@@ -796,8 +796,8 @@ extern "C" int sdv2_swa_attn_default_splits(int32_t rows, int32_t q_tokens, int3
   if (rows <= 0 || q_tokens <= 0 || heads <= 0 || max_seq_len <= 0) return 1;
   // One workgroup per CU.  With s key-range splits there are qwork * s
   // workgroups; they run in ceil(qwork * s / 256) rounds, each as long as one
-  // workgroup's tile count (padded to a multiple of three) plus a fixed start /
-  // end cost of about three tile times.  Writing and merging the fp32 partial
+  // workgroup's tile count plus a fixed start / end cost of about three tile
+  // times.  Writing and merging the fp32 partial
   // results costs roughly one tile time per 7 MB per split.  Constants fitted
   // to measurements on the five benchmark shapes.
   const int64_t qwork = (int64_t)rows * heads * ((q_tokens + kQTile - 1) / kQTile);
@@ -809,8 +809,7 @@ extern "C" int sdv2_swa_attn_default_splits(int32_t rows, int32_t q_tokens, int3
     const int per = (ntiles + sp - 1) / sp;
     if (sp > 1 && per < 6) break;
     const int64_t rounds = (qwork * sp + kCuSlots - 1) / kCuSlots;
-    const int padded = (per + 2) / 3 * 3;
-    const double cost = (double)rounds * (padded + 3) + (sp > 1 ? sp * partial_tiles : 0.0);
+    const double cost = (double)rounds * (per + 3) + (sp > 1 ? sp * partial_tiles : 0.0);
     if (cost < best_cost - 1e-9) { best_cost = cost; best = sp; }
   }
   return best;
