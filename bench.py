@@ -49,6 +49,8 @@ def parse_args():
     ap.add_argument("--cpu-layers", type=int, default=2)
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="only run the library's plain copy kernel on MIB mebibytes (counter calibration)")
+    ap.add_argument("--fill-phase", action="store_true",
+                    help="also time every chunk of a fresh stream while its ring fills (reported apart)")
     ap.add_argument("--skip-mfma-reference", action="store_true",
                     help="do not time the vendor bf16 GEMM that shows what this box sustains on MFMA")
     return ap.parse_args()
@@ -143,12 +145,17 @@ def gpu_bench(args, w):
         step()
     torch.cuda.synchronize()
 
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
     t0 = time.perf_counter()
-    for _ in range(args.steps):
+    for i in range(args.steps):
+        marks[i].record()
         step()
+    marks[args.steps].record()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
+    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+    ms_median = per_step[len(per_step) // 2]
 
     # instrumented pass over the same steps: per-kernel durations
     timers = []
@@ -159,8 +166,28 @@ def gpu_bench(args, w):
     t_attn = sum(e[1].elapsed_time(e[2]) for e in timers) / len(timers)
     t_merge = sum(e[2].elapsed_time(e[3]) for e in timers) / len(timers)
     splits = args.num_splits or _capi.lib().sdv2_swa_attn_default_splits(B, S, H, w.cache_tokens)
+    fill_ms = None
+    if args.fill_phase:
+        # a second, fresh stream from chunk 0: latency of every chunk while the ring fills
+        f_caches = ring.new_kv_cache(w.layers, 1, w.cache_tokens, H, total_steps=1, dtype=w.dtype, device=dev)
+        f_paths = [RingKVPath(sink_size=w.sink_size, adapt_sink_thr=-1) for _ in range(w.layers)]
+        fill_ms = []
+        for call in range(fill_calls):
+            if call == 1 and B > 1:
+                ring.replicate_for_stream_batch(f_caches, B)
+            rows = 1 if (call == 0 and B > 1) else B
+            starts = [min(c, max_chunk) * S for c in workloads.row_chunks(w, call)][:rows]
+            torch.cuda.synchronize()
+            c0 = time.perf_counter()
+            for layer in range(w.layers):
+                q, k, v = qkv[layer]
+                f_paths[layer].attend(q[:rows], k[:rows], v[:rows], grid_sizes[:rows], freqs, f_caches[layer], starts)
+            torch.cuda.synchronize()
+            fill_ms.append((time.perf_counter() - c0) * 1e3)
     return {
         "ms_per_step": ms_per_step,
+        "ms_median": ms_median,
+        "fill_ms": fill_ms,
         "append_ms": t_append,
         "attn_ms": t_attn,
         "merge_ms": t_merge,
@@ -289,6 +316,7 @@ def main():
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": g["ms_per_step"],
+        "ms_per_step_median": g["ms_median"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -324,6 +352,8 @@ def main():
         },
         "kernel_ms_per_layer": {"append": g["append_ms"], "attn": g["attn_ms"], "merge": g["merge_ms"]},
     }
+    if g["fill_ms"] is not None:
+        result["fill_phase_ms_per_chunk"] = [round(x, 4) for x in g["fill_ms"]]
     if not args.skip_mfma_reference:
         ref = mfma_reference()
         ref["attention_vs_random"] = achieved_tflops / ref["random"]
