@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define SDV2KV_ABI_VERSION 1
+#define SDV2KV_ABI_VERSION 2
 #define SDV2_HEAD_DIM 128      /* causal_stream_inference.py:99-100 fixes 128 */
 #define SDV2_MAX_ROWS 16       /* rows (B) per sdv2_kv_append_rope call       */
 #define SDV2_MAX_SINK_FRAMES 16 /* sink frames per sdv2_sink_similarity call  */
@@ -120,8 +120,9 @@ int sdv2_kv_append_rope(const sdv2_append_params* p);
  * v_cache=, cache_seqlens=) as called at models/wan/causal_model.py:353-358
  * and its SDPA fallback attention_with_kvcache_fallback (:111-157):
  *   out[i] = softmax(q[i] k_cache[i,:seq_lens[i]]^T / sqrt(128)) v_cache[i,:seq_lens[i]]
- * with no mask inside the chunk (causal=False) and keys at or beyond
- * seq_lens[i] ignored.  bf16 in, fp32 accumulation, bf16 out.
+ * with no mask inside the chunk (causal=False) unless one is asked for (see
+ * mask_block_tokens) and keys at or beyond seq_lens[i] ignored.  bf16 in, fp32
+ * accumulation, bf16 out.
  *
  * Long caches are split over key ranges to fill the 256 CUs; partial results
  * go through `workspace` (size from sdv2_swa_attn_workspace_bytes) and are
@@ -148,6 +149,17 @@ typedef struct sdv2_attn_params {
   void* workspace;             /* device scratch, 256-byte aligned             */
   size_t workspace_bytes;
   void* stream;                /* hipStream_t                                  */
+  /* Optional block-causal mask INSIDE the chunk.  The reference's cache path
+   * applies none (the chunk is one block); its cache-less path masks with
+   * kv_idx < ends[q_idx] (causal_model.py:670-686).  With mask_block_tokens =
+   * b in (0, S) and the chunk's own keys at cache positions
+   * [chunk_key_start[i], chunk_key_start[i] + S), query token t of row i does
+   * not see the chunk's later blocks, i.e. cache positions
+   * [chunk_key_start[i] + (t / b + 1) * b, chunk_key_start[i] + S); everything
+   * else in the cache is older and stays visible.  0 (or b >= S) = no mask.  */
+  int32_t mask_block_tokens;
+  const int32_t* chunk_key_start;  /* device int32 [B], each in [0, L - S]; may be */
+                                   /* NULL when the mask is off                    */
 } sdv2_attn_params;
 
 /* number of key-range splits the library would pick for this shape */

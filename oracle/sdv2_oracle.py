@@ -119,12 +119,45 @@ def causal_rope_apply(
 # KV-cache attention (the operator the flash kernel replaces)
 # --------------------------------------------------------------------------
 
+def chunk_block_mask(q_tokens: int, keys: int, chunk_start: int, block_tokens: int) -> torch.Tensor:
+    """Boolean [q_tokens, keys], True = visible: the block-causal rule of the
+    cache-less path, kv_idx < ends[q_idx] (causal_model.py:670-686), carried
+    over to cache positions.  The chunk's own keys sit at
+    [chunk_start, chunk_start + q_tokens); whatever else the cache holds is
+    older than the chunk and visible; inside the chunk query t sees its own
+    block and the earlier ones, i.e. not [chunk_start + (t // b + 1) * b,
+    chunk_start + q_tokens)."""
+    t = torch.arange(q_tokens).unsqueeze(1)
+    key = torch.arange(keys).unsqueeze(0)
+    hidden_from = chunk_start + (t // block_tokens + 1) * block_tokens
+    return ~((key >= hidden_from) & (key < chunk_start + q_tokens))
+
+
+def _sdpa_rows(q, k_cache, v_cache, lens, out_dtype, widen, chunk_start, block_tokens):
+    rows = []
+    for b, n in enumerate(lens):
+        qq, kk, vv = widen(
+            q[b:b + 1].transpose(1, 2),
+            k_cache[b:b + 1, :n].transpose(1, 2),
+            v_cache[b:b + 1, :n].transpose(1, 2),
+        )
+        mask = None
+        if block_tokens:
+            mask = chunk_block_mask(q.shape[1], n, int(chunk_start[b]), block_tokens)
+        o = F.scaled_dot_product_attention(qq, kk, vv, attn_mask=mask, dropout_p=0.0, is_causal=False)
+        rows.append(o.transpose(1, 2) if out_dtype is None else o.transpose(1, 2).to(out_dtype))
+    return torch.cat(rows, dim=0).contiguous()
+
+
 def attention_with_kvcache(
-    q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, cache_seqlens: torch.Tensor
+    q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, cache_seqlens: torch.Tensor,
+    chunk_start: Optional[Sequence[int]] = None, block_tokens: int = 0,
 ) -> torch.Tensor:
     """softmax(q k^T / sqrt(D)) v over the first cache_seqlens[b] keys of each
-    row, no mask inside the chunk (causal_model.py:111-157).  bf16/fp16 inputs
-    are up-cast to fp32 on the CPU exactly as the reference fallback does."""
+    row, no mask inside the chunk (causal_model.py:111-157) unless
+    ``block_tokens`` asks for the block-causal one (see chunk_block_mask).
+    bf16/fp16 inputs are up-cast to fp32 on the CPU exactly as the reference
+    fallback does."""
     out_dtype = q.dtype
 
     def widen(*ts):
@@ -133,36 +166,21 @@ def attention_with_kvcache(
         return ts
 
     span = k_cache.shape[1]
-    if bool(torch.all(cache_seqlens == span)):
+    if not block_tokens and bool(torch.all(cache_seqlens == span)):
         qq, kk, vv = widen(q.transpose(1, 2), k_cache.transpose(1, 2), v_cache.transpose(1, 2))
         o = F.scaled_dot_product_attention(qq, kk, vv, attn_mask=None, dropout_p=0.0, is_causal=False)
         return o.transpose(1, 2).to(out_dtype).contiguous()
-
-    rows = []
-    for b, n in enumerate(cache_seqlens.tolist()):
-        qq, kk, vv = widen(
-            q[b:b + 1].transpose(1, 2),
-            k_cache[b:b + 1, :n].transpose(1, 2),
-            v_cache[b:b + 1, :n].transpose(1, 2),
-        )
-        o = F.scaled_dot_product_attention(qq, kk, vv, attn_mask=None, dropout_p=0.0, is_causal=False)
-        rows.append(o.transpose(1, 2).to(out_dtype))
-    return torch.cat(rows, dim=0).contiguous()
+    return _sdpa_rows(q, k_cache, v_cache, cache_seqlens.tolist(), out_dtype, widen, chunk_start, block_tokens)
 
 
 def attention_fp32_reference(
-    q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, cache_seqlens: Sequence[int]
+    q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, cache_seqlens: Sequence[int],
+    chunk_start: Optional[Sequence[int]] = None, block_tokens: int = 0,
 ) -> torch.Tensor:
     """fp32 result (not rounded to the input dtype) — the yardstick the
     2e-2 / 2e-3 tolerances are stated against."""
-    rows = []
-    for b, n in enumerate(cache_seqlens):
-        qq = q[b:b + 1].float().transpose(1, 2)
-        kk = k_cache[b:b + 1, :n].float().transpose(1, 2)
-        vv = v_cache[b:b + 1, :n].float().transpose(1, 2)
-        o = F.scaled_dot_product_attention(qq, kk, vv, attn_mask=None, dropout_p=0.0, is_causal=False)
-        rows.append(o.transpose(1, 2))
-    return torch.cat(rows, dim=0).contiguous()
+    return _sdpa_rows(q, k_cache, v_cache, list(cache_seqlens), None, lambda *ts: tuple(t.float() for t in ts),
+                      chunk_start, block_tokens)
 
 
 # --------------------------------------------------------------------------
@@ -218,6 +236,8 @@ class RingAttentionOracle:
         self.sink_size = sink_size
         self.adapt_sink_thr = adapt_sink_thr
         self.evict_idx: Optional[List[List[int]]] = None
+        # None = the chunk is one block (reference cache path); n = blocks of n frames
+        self.block_frames: Optional[int] = None
         # what the last call did, for tests: per row (dst_start, dst_end)
         self.last_writes: List[Tuple[int, int]] = []
         # per row the averaged similarities of the adaptive sink check, or None
@@ -310,8 +330,12 @@ class RingAttentionOracle:
         if with_attention:
             lens = torch.tensor(seq_lens, dtype=torch.int32)
             span = int(lens.max().item())
+            block_tokens = 0
+            if self.block_frames is not None and self.block_frames * frame_tokens < n_new:
+                block_tokens = self.block_frames * frame_tokens
             out = attention_with_kvcache(
-                roped_q, kv_cache["k"][:, :span], kv_cache["v"][:, :span], lens
+                roped_q, kv_cache["k"][:, :span], kv_cache["v"][:, :span], lens,
+                [a for a, _ in self.last_writes], block_tokens,
             )
         return out, roped_q, seq_lens
 

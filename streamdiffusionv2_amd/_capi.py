@@ -11,7 +11,7 @@ from typing import Optional
 
 LIB_PATH = Path(__file__).resolve().parent / "_lib" / "libsdv2kv.so"
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 HEAD_DIM = 128
 MAX_ROWS = 16
 
@@ -80,6 +80,8 @@ class AttnParams(C.Structure):
         ("workspace", C.c_void_p),
         ("workspace_bytes", C.c_size_t),
         ("stream", C.c_void_p),
+        ("mask_block_tokens", C.c_int32),
+        ("chunk_key_start", C.c_void_p),
     ]
 
 

@@ -73,6 +73,11 @@ class RingKVPath:
 
     # 0 lets the library choose how many key ranges an attention call is split into
     num_splits = 0
+    # None: the chunk is one block, nothing is masked inside it (what the
+    # reference's cache path does).  n: blocks of n latent frames, a query sees
+    # the cache and its chunk's blocks up to its own (the cache-less path's
+    # kv_idx < ends[q_idx], causal_model.py:670-686).
+    block_frames: Optional[int] = None
 
     def _layer_launcher(self, q, k, v, kv_cache, table, grid):
         """The cached launch descriptors for this layer, rebuilt when the
@@ -134,12 +139,15 @@ class RingKVPath:
             # lengths are a handful of host ints, shipped asynchronously
             seq = torch.tensor(plan.new_local_end, dtype=torch.int32).to(q.device, non_blocking=True)
         self.last_plan = plan
+        mask_tokens = 0
+        if self.block_frames is not None and self.block_frames * frame_tokens < q.shape[1]:
+            mask_tokens = self.block_frames * frame_tokens
 
         if q.dtype == torch.bfloat16 and rows <= ops._capi.MAX_ROWS:
             # steady-state fast path: launch descriptors are built once per
             # (cache, shape) and only patched per call
             launcher = self._layer_launcher(q, k, v, kv_cache, table, (f, h, w))
-            out = launcher.launch(q, k, v, [c // frame_tokens for c in starts], plan, seq)
+            out = launcher.launch(q, k, v, [c // frame_tokens for c in starts], plan, seq, mask_tokens)
             if return_roped_query:
                 return out, launcher.roped_q.clone()
             return out
@@ -152,14 +160,15 @@ class RingKVPath:
             new_global_end=plan.new_global_end,
             new_local_end=plan.new_local_end,
         )
+        mask = dict(chunk_key_start=list(plan.dst_start), mask_block_tokens=mask_tokens) if mask_tokens else {}
         if roped_q.dtype == torch.bfloat16:
-            out = ops.swa_attention(roped_q, kv_cache["k"][:, :span], kv_cache["v"][:, :span], seq)
+            out = ops.swa_attention(roped_q, kv_cache["k"][:, :span], kv_cache["v"][:, :span], seq, **mask)
         else:
             # fp32 storage is a plumbing mode (the reference's CPU-runnable
             # configuration): RoPE, cache and indices stay fp32 and bit-exact,
             # the attention kernel computes in bf16 on down-cast copies.
             out = ops.swa_attention(
-                roped_q.bfloat16(), kv_cache["k"][:, :span].bfloat16(), kv_cache["v"][:, :span].bfloat16(), seq
+                roped_q.bfloat16(), kv_cache["k"][:, :span].bfloat16(), kv_cache["v"][:, :span].bfloat16(), seq, **mask
             ).to(roped_q.dtype)
         if return_roped_query:
             return out, roped_q

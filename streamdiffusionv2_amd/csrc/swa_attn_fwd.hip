@@ -27,8 +27,8 @@
 // maximum: the weights stay in fp32 / bf16 range as long as the scaled scores
 // stay within about +-100 in log2 units, which every sane attention input
 // does, and the result is mathematically the same.  Each wave checks its row
-// sums every slot; if any leaves [2^-100, 2^100] (or is NaN) the workgroup
-// finishes the fast pass, throws its result away and recomputes with the
+// sums after its last tile; if any left [2^-100, 2^100] (or is NaN) the
+// workgroup throws the result away and recomputes with the
 // conventional running-maximum recurrence (slow, exact for any finite input).
 //
 // LDS tile layout: row r (key) holds sixteen 16-byte chunks; chunk c is stored
@@ -87,6 +87,8 @@ struct AttnKernelArgs {
   sdv2_stride3 q_st, k_st, v_st, o_st;
   int32_t rows, q_tokens, heads, max_seq_len, num_splits;
   float scale_log2;            // softmax_scale * log2(e)
+  int32_t mask_block_tokens;   // 0 = no mask inside the chunk
+  const int32_t* chunk_start;  // device [rows]: cache position of the chunk's own first key
   float* part_o;               // [split][row][head][q][128] fp32, normalised
   float* part_lse;             // [split][row][head][q]      log2 sum exp
 };
@@ -255,13 +257,19 @@ struct LaneConst {
   uint32_t v_addr[4][2];  // V^T fragment of d block db, key sub-quad j, within a 16-key step
   float c2;               // softmax scale * log2(e)
   int hf;                 // lane / 32
+  // block-causal mask inside the chunk: keys [m_lo, m_hi) are the chunk's own
+  // later blocks, hidden from this lane's query; [wg_m_lo, m_hi) is the union
+  // over the workgroup's queries (wave-uniform).  Empty when the mask is off.
+  int m_lo[kQB];
+  int m_hi;
+  int wg_m_lo;
 };
 
-__device__ __forceinline__ void mask_block(f32x16& s, int key0, int seq, int hf) {
+__device__ __forceinline__ void mask_block(f32x16& s, int key0, int seq, int hf, int m_lo, int m_hi) {
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
     const int key = key0 + 8 * (i >> 2) + 4 * hf + (i & 3);
-    if (key >= seq) s[i] = -INFINITY;
+    if (key >= seq || (key >= m_lo && key < m_hi)) s[i] = -INFINITY;
   }
 }
 
@@ -278,7 +286,7 @@ __device__ __forceinline__ void mask_block(f32x16& s, int key0, int seq, int hf)
 // s[j&1], P(j) in p[j&1]; with the slot parity a template argument this is
 // pure register naming.
 // ---------------------------------------------------------------------------
-template <int kPar, int kKOff, int kVOff, bool kDoS, bool kDoPV, bool kDoSM>
+template <bool kMask, int kPar, int kKOff, int kVOff, bool kDoS, bool kDoPV, bool kDoSM>
 __device__ __forceinline__ void slot(const LaneConst& c, const bf16x8 (&qf)[kQB][8], f32x16 (&s)[2][kQB],
                                      u32x4 (&p)[2][kQB][2], f32x16 (&oacc)[kQB][4], float (&l)[kQB],
                                      int key0, int key_end) {
@@ -306,14 +314,23 @@ __device__ __forceinline__ void slot(const LaneConst& c, const bf16x8 (&qf)[kQB]
   static_for<kAhead>(request);
 
   if constexpr (kDoSM) {
-    // the last, partial tile and the padding tiles behind it.  The test value
+    // the last, partial tile, and blocks that hold the chunk's own later
+    // frames when a mask inside the chunk is asked for.  The test value
     // goes through an empty asm so that the compiler cannot fold this uniform,
     // rarely taken branch into the per-lane compares and hoist those.
-    int beyond = key0 + 32 - key_end;
-    asm volatile("" : "+s"(beyond));
-    if (beyond > 0) {
+    // > 0 when the block reaches past key_end or (with the mask inside the chunk
+    // compiled in) overlaps [wg_m_lo, m_hi); integer min / max keep the test in
+    // scalar registers
+    int masked = key0 + 32 - key_end;
+    if constexpr (kMask) {
+      const int into_hidden = key0 + 32 - c.wg_m_lo < c.m_hi - key0 ? key0 + 32 - c.wg_m_lo : c.m_hi - key0;
+      masked = masked > into_hidden ? masked : into_hidden;
+    }
+    asm volatile("" : "+s"(masked));
+    if (masked > 0) {
 #pragma unroll
-      for (int qb = 0; qb < kQB; ++qb) mask_block(s_cur[qb], key0, key_end, c.hf);
+      for (int qb = 0; qb < kQB; ++qb)
+        mask_block(s_cur[qb], key0, key_end, c.hf, kMask ? c.m_lo[qb] : 0x7fffffff, kMask ? c.m_hi : 0);
     }
   }
   __builtin_amdgcn_sched_barrier(0);
@@ -417,7 +434,8 @@ __device__ __forceinline__ void exact_pass(const AttnKernelArgs& a, const LaneCo
               lds + (c.k_addr[ks] - lds_addr0) + kLdsK(0) + kb * 32 * 256);
           sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][ks], sacc[kb], 0, 0, 0);
         }
-        if (key0 + kb * 32 + 32 > seq) mask_block(sacc[kb], key0 + kb * 32, seq, c.hf);
+        if (key0 + kb * 32 + 32 > seq || (key0 + kb * 32 + 32 > c.wg_m_lo && key0 + kb * 32 < c.m_hi))
+          mask_block(sacc[kb], key0 + kb * 32, seq, c.hf, c.m_lo[qb], c.m_hi);
       }
       float mloc = sacc[0][0];
 #pragma unroll
@@ -425,9 +443,10 @@ __device__ __forceinline__ void exact_pass(const AttnKernelArgs& a, const LaneCo
 #pragma unroll
         for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, sacc[kb][i]);
       mloc = half_max(mloc);
-      const float m_new = fmaxf(m_run[qb], mloc);      // finite: every tile has a valid key
-      const float alpha = __builtin_amdgcn_exp2f((m_run[qb] - m_new) * c.c2);
-      const float mc = m_new * c.c2;
+      const float m_new = fmaxf(m_run[qb], mloc);
+      // -inf only while every key so far was masked for this query: then nothing has been summed yet
+      const float alpha = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f((m_run[qb] - m_new) * c.c2);
+      const float mc = m_new == -INFINITY ? 0.0f : m_new * c.c2;
       m_run[qb] = m_new;
       float psum = 0.f;
       bf16x8 pf[2][2];
@@ -465,6 +484,7 @@ __device__ __forceinline__ void exact_pass(const AttnKernelArgs& a, const LaneCo
   }
 }
 
+template <bool kMask>
 __global__ __launch_bounds__(kThreads, 1)
 void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -556,6 +576,19 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   LaneConst c;
   c.c2 = a.scale_log2;
   c.hf = hf;
+  if (kMask && a.mask_block_tokens > 0) {
+    const int bt = a.mask_block_tokens;
+    const int first = a.chunk_start[row];
+    c.m_hi = __builtin_amdgcn_readfirstlane(first + a.q_tokens);
+    c.wg_m_lo = __builtin_amdgcn_readfirstlane(first + ((qtile * kQTile) / bt + 1) * bt);
+#pragma unroll
+    for (int qb = 0; qb < kQB; ++qb) c.m_lo[qb] = first + (q_row[qb] / bt + 1) * bt;
+  } else {
+    c.m_hi = 0;
+    c.wg_m_lo = 0x7fffffff;
+#pragma unroll
+    for (int qb = 0; qb < kQB; ++qb) c.m_lo[qb] = 0x7fffffff;
+  }
   {
     // K (A operand): key = lane%32 of the block, chunk = 2*ks + hf
     const int r = lane & 31;
@@ -616,17 +649,26 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   // whatever finite data the buffers still hold.  In the first slot P(-1) is
   // zero likewise.
   const int key_end = seq < tile_end * kKTile ? seq : tile_end * kKTile;
+  // Checked once, after the last tile: a sum that overflowed stays inf or NaN, one
+  // that underflowed stays tiny.  With the mask inside the chunk a sum of exactly
+  // zero is legitimate when every key of this workgroup's range is hidden from
+  // the lane's query (its split then contributes nothing).
   auto row_sums_unsafe = [&]() {
     bool bad = false;
 #pragma unroll
-    for (int qb = 0; qb < kQB; ++qb) bad |= !(l_run[qb] >= 0x1p-100f && l_run[qb] <= 0x1p100f);
+    for (int qb = 0; qb < kQB; ++qb) {
+      bool ok = l_run[qb] >= 0x1p-100f && l_run[qb] <= 0x1p100f;
+      if constexpr (kMask)
+        ok |= l_run[qb] == 0.f && tile_begin * kKTile >= c.m_lo[qb] && key_end <= c.m_hi;
+      bad |= !ok;
+    }
     return __builtin_amdgcn_ballot_w64(bad) != 0;
   };
   auto do_tile = [&](auto buf_c, int T) {
     constexpr int kB = decltype(buf_c)::value;              // T % 3
     constexpr int kBNext = (kB + 1) % kStages, kBPrev = (kB + 2) % kStages;
     const int key0 = (tile_begin + T) * kKTile;
-    slot<0, kLdsK(kB) + 32 * 256, kLdsVRel(kBPrev) + 32 * 256, true, true, true>(c, qf, s, p, oacc, l_run, key0,
+    slot<kMask, 0, kLdsK(kB) + 32 * 256, kLdsVRel(kBPrev) + 32 * 256, true, true, true>(c, qf, s, p, oacc, l_run, key0,
                                                                                 key_end);
     if (T + 3 < n) {
       __builtin_amdgcn_s_waitcnt(0x0F78);   // vmcnt(8)
@@ -636,8 +678,7 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
     __syncthreads();
     if (T + 3 < n) issue_k(T + 3, kB);
     if (T + 2 < n) issue_v(T + 2, kBPrev);
-    slot<1, kLdsK(kBNext), kLdsVRel(kB), true, true, true>(c, qf, s, p, oacc, l_run, key0 + 32, key_end);
-    unsafe |= row_sums_unsafe();
+    slot<kMask, 1, kLdsK(kBNext), kLdsVRel(kB), true, true, true>(c, qf, s, p, oacc, l_run, key0 + 32, key_end);
   };
   using B0 = std::integral_constant<int, 0>;
   using B1 = std::integral_constant<int, 1>;
@@ -647,7 +688,7 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();        // the first tiles and the Q fragments have arrived
     // S(0) alone fills the pipeline
-    slot<1, kLdsK(0), 0, true, false, false>(c, qf, s, p, oacc, l_run, 0, key_end);
+    slot<kMask, 1, kLdsK(0), 0, true, false, false>(c, qf, s, p, oacc, l_run, 0, key_end);
     // Three tiles per trip, one per buffer; the last trip stops after the last
     // real tile.  The skipped tiles sit behind uniform branches that no value
     // is changed on, so the accumulators stay where they are on either way.
@@ -668,9 +709,10 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
       for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int j = 0; j < 2; ++j) cf.v_addr[db][j] = c.v_addr[db][j] + shift;
-      slot<0, 0, kLdsVRel(2) + 32 * 256, false, true, false>(cf, qf, s, p, oacc, l_run, 0, key_end);
+      slot<kMask, 0, 0, kLdsVRel(2) + 32 * 256, false, true, false>(cf, qf, s, p, oacc, l_run, 0, key_end);
     }
     mfma_drain<0>(oacc, s);
+    unsafe = row_sums_unsafe();
 
     // Did any wave of the workgroup see an unsafe row sum?  (LDS is free now.)
     __syncthreads();
@@ -854,6 +896,13 @@ extern "C" int sdv2_swa_attn_fwd(const sdv2_attn_params* p) {
   a.num_splits = splits;
   const float scale = p->softmax_scale > 0.f ? p->softmax_scale : 0.08838834764831845f;  // 1/sqrt(128)
   a.scale_log2 = scale * kLog2e;
+  if (p->mask_block_tokens < 0) return SDV2_ERR_INVALID_ARG;
+  if (p->mask_block_tokens > 0 && p->mask_block_tokens < p->q_tokens) {
+    // a block as long as the chunk hides nothing: only shorter blocks switch the mask on
+    if (!p->chunk_key_start) return SDV2_ERR_INVALID_ARG;
+    a.chunk_start = p->chunk_key_start;
+    a.mask_block_tokens = p->mask_block_tokens;
+  }
 
   if (splits > 1) {
     const size_t need = sdv2_swa_attn_workspace_bytes(p->rows, p->q_tokens, p->heads, p->max_seq_len, splits);
@@ -870,11 +919,21 @@ extern "C" int sdv2_swa_attn_fwd(const sdv2_attn_params* p) {
   if (items > (1 << 28)) return SDV2_ERR_INVALID_ARG;
   dim3 grid((unsigned)(8 * ((items + 7) / 8)));
   if (p->stages != SDV2_STAGE_MERGE) {
-    // 96 KB of LDS is more than the static limit: ask for it once per process
-    static const hipError_t lds_attr = hipFuncSetAttribute(
-        reinterpret_cast<const void*>(swa_attn_fwd_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    // 96 KB of LDS is more than the static limit: ask for it once per process.
+    // The kernel exists twice: the mask inside the chunk costs the plain
+    // variant about 2 % even when it is off, so it gets its own code.
+    static const hipError_t lds_attr = [] {
+      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(swa_attn_fwd_kernel<false>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+      return e != hipSuccess ? e
+                             : hipFuncSetAttribute(reinterpret_cast<const void*>(swa_attn_fwd_kernel<true>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    }();
     if (lds_attr != hipSuccess) return SDV2_ERR_LAUNCH;
-    hipLaunchKernelGGL(swa_attn_fwd_kernel, grid, dim3(kThreads), kLdsBytes, stream, a);
+    if (a.mask_block_tokens > 0)
+      hipLaunchKernelGGL(swa_attn_fwd_kernel<true>, grid, dim3(kThreads), kLdsBytes, stream, a);
+    else
+      hipLaunchKernelGGL(swa_attn_fwd_kernel<false>, grid, dim3(kThreads), kLdsBytes, stream, a);
     if (hipGetLastError() != hipSuccess) return SDV2_ERR_LAUNCH;
   }
   if (splits > 1 && p->stages != SDV2_STAGE_PARTIAL) {

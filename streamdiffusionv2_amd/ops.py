@@ -171,6 +171,21 @@ def _workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
     return ws
 
 
+def chunk_starts_tensor(starts, rows: int, q_tokens: int, max_seq_len: int, dev) -> torch.Tensor:
+    """Per-row cache position of the chunk's own keys as the int32 device
+    tensor the attention kernel reads; host values are range-checked here."""
+    if isinstance(starts, torch.Tensor):
+        if starts.dtype != torch.int32 or starts.numel() != rows or starts.device != dev or not starts.is_contiguous():
+            raise RuntimeError("chunk_key_start must be a contiguous int32 device tensor with one entry per row")
+        return starts
+    if starts is None or len(starts) != rows:
+        raise RuntimeError("mask_block_tokens needs chunk_key_start with one entry per row")
+    for x in starts:
+        if x < 0 or x + q_tokens > max_seq_len:
+            raise RuntimeError(f"chunk_key_start {x} puts the chunk outside the {max_seq_len}-key view")
+    return torch.tensor([int(x) for x in starts], dtype=torch.int32).to(dev, non_blocking=True)
+
+
 def swa_attention(
     q: torch.Tensor,
     k_cache: torch.Tensor,
@@ -181,11 +196,17 @@ def swa_attention(
     softmax_scale: Optional[float] = None,
     workspace: Optional[torch.Tensor] = None,
     stages: int = _capi.STAGE_ALL,
+    chunk_key_start: Optional[torch.Tensor] = None,
+    mask_block_tokens: int = 0,
 ) -> torch.Tensor:
     """out[b] = softmax(q[b] k_cache[b,:seq_lens[b]]^T * scale) v_cache[b,:seq_lens[b]].
 
     q [B,S,H,128] bf16; k_cache/v_cache [B,L,H,128] bf16 views with any row /
     token / head strides; seq_lens int32 [B] on the device (None = L).
+    With ``mask_block_tokens`` = b in (0, S) and ``chunk_key_start`` (int32 [B]
+    on the device, or host ints: where each row's own chunk sits in the cache)
+    query token t does not see the chunk's later blocks
+    [start + (t // b + 1) * b, start + S).
     """
     dev = _require_gpu(q, k_cache, v_cache, seq_lens, out, workspace)
     if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
@@ -223,6 +244,10 @@ def swa_attention(
         p.workspace = workspace.data_ptr()
         p.workspace_bytes = workspace.numel() * workspace.element_size()
     p.stream = _stream_ptr(dev)
+    if mask_block_tokens:
+        chunk_key_start = chunk_starts_tensor(chunk_key_start, rows, q_tokens, max_seq_len, dev)
+        p.mask_block_tokens = int(mask_block_tokens)
+        p.chunk_key_start = chunk_key_start.data_ptr()
     with torch.cuda.device(dev):
         _capi.check(lib.sdv2_swa_attn_fwd(C.byref(p)), "sdv2_swa_attn_fwd")
     return out
@@ -368,10 +393,15 @@ class LayerLauncher:
         return self.cache_sig == (kc.data_ptr(), vc.data_ptr(), tuple(kc.shape), tuple(kc.stride()), tuple(vc.stride()),
                                   kv_cache["global_end_index"].data_ptr(), kv_cache["local_end_index"].data_ptr())
 
-    def patch(self, q, k, v, start_frames, plan, seq_lens: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def patch(self, q, k, v, start_frames, plan, seq_lens: Optional[torch.Tensor] = None,
+              mask_block_tokens: int = 0) -> torch.Tensor:
         """Fill in what changes from call to call and allocate the output
         [rows, S, H, 128]; nothing is launched."""
         ap, at = self.ap, self.at
+        at.mask_block_tokens = mask_block_tokens
+        if mask_block_tokens:
+            self.chunk_starts = chunk_starts_tensor(plan.dst_start, self.rows, self.tokens, plan.max_seq_len, self.dev)
+            at.chunk_key_start = self.chunk_starts.data_ptr()
         for i in range(self.rows):
             self.sf[i] = start_frames[i]
             self.ds[i] = plan.dst_start[i]
@@ -409,10 +439,11 @@ class LayerLauncher:
         self.at.stages = stages
         _capi.check(self.lib.sdv2_swa_attn_fwd(self.at_ref), "sdv2_swa_attn_fwd")
 
-    def launch(self, q, k, v, start_frames, plan, seq_lens: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def launch(self, q, k, v, start_frames, plan, seq_lens: Optional[torch.Tensor] = None,
+               mask_block_tokens: int = 0) -> torch.Tensor:
         """Append + attention for one call; returns the attention output
         [rows, S, H, 128].  The roped query stays in ``self.roped_q``."""
-        out = self.patch(q, k, v, start_frames, plan, seq_lens)
+        out = self.patch(q, k, v, start_frames, plan, seq_lens, mask_block_tokens)
         if _current_device_index() != self.dev.index:
             with torch.cuda.device(self.dev):
                 self.run_append()
