@@ -51,6 +51,8 @@ def parse_args():
                     help="only run the library's plain copy kernel on MIB mebibytes (counter calibration)")
     ap.add_argument("--fill-phase", action="store_true",
                     help="also time every chunk of a fresh stream while its ring fills (reported apart)")
+    ap.add_argument("--qk-norm", action="store_true",
+                    help="also time the append with the q/k RMSNorm folded in against torch norms + plain append")
     ap.add_argument("--skip-mfma-reference", action="store_true",
                     help="do not time the vendor bf16 GEMM that shows what this box sustains on MFMA")
     return ap.parse_args()
@@ -223,6 +225,59 @@ def mfma_reference(n=8192, iters=20):
     return out
 
 
+def qk_norm_section(args, w):
+    """Append with the q / k RMSNorm folded in (one kernel) against the same
+    work done as the reference does it (two WanRMSNorm modules in torch, then
+    the plain append kernel).  Times are per layer call, HIP events around a
+    run of calls that rotates over all layers' tensors."""
+    from streamdiffusionv2_amd import ops, ring, workloads
+    from streamdiffusionv2_amd.attention import WanRMSNorm
+
+    dev = torch.device("cuda:0")
+    S, H, B = w.chunk_tokens, w.heads, w.rows
+    layers = min(w.layers, 12)
+    caches = ring.new_kv_cache(layers, 1, w.cache_tokens, H, 1, dtype=w.dtype, device=dev)
+    if B > 1:
+        ring.replicate_for_stream_batch(caches, B)
+    table = ops.device_freqs(build_freqs(), dev)
+    qkv = [tuple(t.to(dev) for t in workloads.make_qkv(w, 0, layer)) for layer in range(layers)]
+    norm_q, norm_k = WanRMSNorm(H * 128, eps=1e-6).to(dev).to(w.dtype), WanRMSNorm(H * 128, eps=1e-6).to(dev).to(w.dtype)
+    weights = (norm_q.weight.detach(), norm_k.weight.detach(), 1e-6)
+    q_out = torch.empty_like(qkv[0][0])
+    starts, dst = [3] * B, [S] * B
+
+    def fused(i):
+        q, k, v = qkv[i % layers]
+        c = caches[i % layers]
+        ops.kv_append_rope(q, k, v, c["k"], c["v"], table, w.grid, starts, dst, q_out=q_out, qk_norm=weights)
+
+    def unfused(i):
+        q, k, v = qkv[i % layers]
+        c = caches[i % layers]
+        with torch.no_grad():
+            qn = norm_q(q.flatten(2)).view_as(q)
+            kn = norm_k(k.flatten(2)).view_as(k)
+        ops.kv_append_rope(qn, kn, v, c["k"], c["v"], table, w.grid, starts, dst, q_out=q_out)
+
+    out = {}
+    n = 4 * layers
+    for name, fn in (("fused_ms", fused), ("torch_norms_plus_append_ms", unfused)):
+        for i in range(layers):
+            fn(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(n):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        out[name] = e0.elapsed_time(e1) / n
+    out["bytes_per_launch"] = w.append_bytes(with_q=True)
+    out["fused_GBps"] = out["bytes_per_launch"] / (out["fused_ms"] * 1e-3) / 1e9
+    out["note"] = "host-inclusive per-call times; the torch path launches about a dozen kernels per call"
+    return out
+
+
 def cpu_baseline(args, w):
     """The CPU oracle (a PyTorch restatement of the reference's op sequence)
     on this box's host cores: a bounded sample of steady-state chunks on a few
@@ -354,6 +409,8 @@ def main():
     }
     if g["fill_ms"] is not None:
         result["fill_phase_ms_per_chunk"] = [round(x, 4) for x in g["fill_ms"]]
+    if args.qk_norm:
+        result["fused_qk_norm"] = qk_norm_section(args, w)
     if not args.skip_mfma_reference:
         ref = mfma_reference()
         ref["attention_vs_random"] = achieved_tflops / ref["random"]

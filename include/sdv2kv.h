@@ -108,6 +108,17 @@ typedef struct sdv2_append_params {
   const int64_t* new_global_end;  /* host [B] values stored by the kernel      */
   const int64_t* new_local_end;   /* host [B]                                  */
   void* stream;                /* hipStream_t                                  */
+  /* Optional: fold the q / k RMSNorm of the projection outputs in (WanRMSNorm,
+   * wan_base/modules/model.py:70-86, applied in qkv_fn, causal_model.py:212-218).
+   * With both weights given, q_in and k_in are the raw projection outputs and
+   *   x' = type_as(float(x) * rsqrt(mean_over_heads*128(float(x)^2) + norm_eps)) * weight
+   * is what gets roped.  Weights have the tensors' dtype, heads * 128 elements.
+   * The mean is an fp32 sum in this kernel's order: against another summation
+   * order the normalised value can differ in its last fp32 bit, which shows as
+   * one storage-type ulp in about one element in 10^5.                        */
+  const void* q_norm_weight;   /* device, or NULL (together with k_norm_weight) */
+  const void* k_norm_weight;
+  float norm_eps;
 } sdv2_append_params;
 
 int sdv2_kv_append_rope(const sdv2_append_params* p);

@@ -115,6 +115,13 @@ def causal_rope_apply(
     return out
 
 
+def wan_rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """WanRMSNorm.forward (wan_base/modules/model.py:77-86) over the last
+    dimension: float32 normalisation, back to x's dtype, times the weight."""
+    xf = x.float()
+    return (xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + eps)).type_as(x) * weight
+
+
 # --------------------------------------------------------------------------
 # KV-cache attention (the operator the flash kernel replaces)
 # --------------------------------------------------------------------------

@@ -64,6 +64,9 @@ class AppendParams(C.Structure):
         ("new_global_end", C.POINTER(C.c_int64)),
         ("new_local_end", C.POINTER(C.c_int64)),
         ("stream", C.c_void_p),
+        ("q_norm_weight", C.c_void_p),
+        ("k_norm_weight", C.c_void_p),
+        ("norm_eps", C.c_float),
     ]
 
 

@@ -79,14 +79,14 @@ class RingKVPath:
     # kv_idx < ends[q_idx], causal_model.py:670-686).
     block_frames: Optional[int] = None
 
-    def _layer_launcher(self, q, k, v, kv_cache, table, grid):
+    def _layer_launcher(self, q, k, v, kv_cache, table, grid, qk_norm=None):
         """The cached launch descriptors for this layer, rebuilt when the
-        cache, the shapes or the grid change."""
+        cache, the shapes, the grid or the norm weights change."""
         launcher = getattr(self, "_launcher", None)
-        if launcher is None or not launcher.matches(q, k, v, kv_cache, table) \
+        if launcher is None or not launcher.matches(q, k, v, kv_cache, table, qk_norm) \
                 or (launcher.ap.grid_f, launcher.ap.grid_h, launcher.ap.grid_w) != tuple(grid):
             launcher = ops.LayerLauncher(kv_cache["k"], kv_cache["v"], kv_cache["global_end_index"],
-                                         kv_cache["local_end_index"], table, grid, q, k, v)
+                                         kv_cache["local_end_index"], table, grid, q, k, v, qk_norm=qk_norm)
             self._launcher = launcher
         if launcher.forced_splits != self.num_splits:
             launcher.forced_splits = self.num_splits
@@ -94,9 +94,11 @@ class RingKVPath:
         return launcher
 
     def attend(self, q, k, v, grid_sizes, freqs, kv_cache, current_start,
-               return_roped_query: bool = False):
+               return_roped_query: bool = False, qk_norm=None):
         """RoPE + ring append + attention for q/k/v [B, S, H, 128]
-        (causal_model.py:250-384)."""
+        (causal_model.py:250-384).  With ``qk_norm`` = (q weight, k weight,
+        eps), q and k are the raw projection outputs and their RMSNorm
+        (qkv_fn, causal_model.py:212-218) runs inside the append kernel."""
         rows = q.shape[0]
         grids = _host_ints(grid_sizes, "grid")
         f, h, w = grids[0], grids[1], grids[2]
@@ -119,6 +121,9 @@ class RingKVPath:
         if self.sink_size * frame_tokens > 0 and self.adapt_sink_thr > -1 and q.shape[1] <= frame_tokens:
             # adaptive sink refresh (causal_model.py:284-299): one fused
             # reduction on the device, one small read-back for all rows
+            if qk_norm is not None:
+                raise RuntimeError("adaptive sink refresh reads the normalised key before the append: "
+                                   "apply the q/k norm outside (qk_norm=None) in this mode")
             if q.shape[1] != frame_tokens:
                 raise RuntimeError(
                     f"adaptive sink refresh needs one-frame chunks ({frame_tokens} tokens), got {q.shape[1]}"
@@ -146,7 +151,7 @@ class RingKVPath:
         if q.dtype == torch.bfloat16 and rows <= ops._capi.MAX_ROWS:
             # steady-state fast path: launch descriptors are built once per
             # (cache, shape) and only patched per call
-            launcher = self._layer_launcher(q, k, v, kv_cache, table, (f, h, w))
+            launcher = self._layer_launcher(q, k, v, kv_cache, table, (f, h, w), qk_norm)
             out = launcher.launch(q, k, v, [c // frame_tokens for c in starts], plan, seq, mask_tokens)
             if return_roped_query:
                 return out, launcher.roped_q.clone()
@@ -159,6 +164,7 @@ class RingKVPath:
             local_end_index=kv_cache["local_end_index"],
             new_global_end=plan.new_global_end,
             new_local_end=plan.new_local_end,
+            qk_norm=qk_norm,
         )
         mask = dict(chunk_key_start=list(plan.dst_start), mask_block_tokens=mask_tokens) if mask_tokens else {}
         if roped_q.dtype == torch.bfloat16:
@@ -186,6 +192,10 @@ class CausalWanSelfAttention(nn.Module, RingKVPath):
         self.window_size = window_size
         self.qk_norm = qk_norm
         self.eps = eps
+
+        # the q / k RMSNorm inside the append kernel (its sum of squares is
+        # taken in another order than torch's, see sdv2_append_params)
+        self.fuse_qk_norm = True
 
         # ring state, same defaults as causal_model.py:177-179
         self.sink_size = 3
@@ -221,10 +231,17 @@ class CausalWanSelfAttention(nn.Module, RingKVPath):
                 "training path (causal_model.py:220-249) is out of scope"
             )
         b, s, n, d = *x.shape[:2], self.num_heads, self.head_dim
-        q = self.norm_q(self.q(x)).view(b, s, n, d)
-        k = self.norm_k(self.k(x)).view(b, s, n, d)
         v = self.v(x).view(b, s, n, d)
-        out = self.attend(q, k, v, grid_sizes, freqs, kv_cache, current_start)
+        adaptive = self.sink_size > 0 and self.adapt_sink_thr > -1
+        if self.qk_norm and self.fuse_qk_norm and not adaptive:
+            # the two RMSNorms run inside the append kernel
+            q, k = self.q(x).view(b, s, n, d), self.k(x).view(b, s, n, d)
+            norm = (self.norm_q.weight.detach(), self.norm_k.weight.detach(), self.eps)
+            out = self.attend(q, k, v, grid_sizes, freqs, kv_cache, current_start, qk_norm=norm)
+        else:
+            q = self.norm_q(self.q(x)).view(b, s, n, d)
+            k = self.norm_k(self.k(x)).view(b, s, n, d)
+            out = self.attend(q, k, v, grid_sizes, freqs, kv_cache, current_start)
         return self.o(out.flatten(2))
 
 

@@ -14,6 +14,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "sdv2kv.h"
 #include "sdv2kv_internal.h"
 #include "rope_device.h"
@@ -33,6 +35,9 @@ struct AppendKernelArgs {
   void* v_cache;
   sdv2_stride3 q_in_st, k_in_st, v_in_st, q_out_st, k_st, v_st;
   const double2* freqs;
+  const void* q_norm_w;                     // RMSNorm weights over heads * 128, or null
+  const void* k_norm_w;
+  float norm_eps;
   int64_t* global_end;
   int64_t* local_end;
   int32_t tokens, heads, grid_w, frame_tokens;
@@ -97,6 +102,111 @@ void kv_append_rope_kernel(const AppendKernelArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Append with the q / k RMSNorm of the projection outputs folded in
+// (WanRMSNorm, wan_base/modules/model.py:70-86, as applied in qkv_fn,
+// causal_model.py:212-218): y = type_as(x.float() * rsqrt(mean(x^2) + eps)) *
+// weight over the full heads * 128 vector of a token, then RoPE and the
+// scatter as above.  One wave per token: lane l owns the 8-element slice
+// l % 16 of heads 4 * j + l / 16 (j = 0, 1, ...), keeps its q / k slices in
+// registers between the sum of squares and the write, and the wave reduces the
+// two sums with cross-lane adds in a fixed order.  Rounding steps are the
+// reference's: normalised value to the storage type, times weight to the
+// storage type, rotation in double to float to the storage type.
+// ---------------------------------------------------------------------------
+constexpr int kNormMaxSteps = 16;           // heads <= 64
+
+template <typename T>
+__device__ __forceinline__ float to_storage(float x);
+template <>
+__device__ __forceinline__ float to_storage<uint16_t>(float x) {
+  return sdv2::bf16_bits_to_f32(sdv2::f32_to_bf16_rne(x));
+}
+template <>
+__device__ __forceinline__ float to_storage<float>(float x) { return x; }
+
+template <typename T>
+__device__ __forceinline__ sdv2::Vec8<T> normalise(const sdv2::Vec8<T>& x, float r, const sdv2::Vec8<T>& w) {
+  sdv2::Vec8<T> y;
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const float a = to_storage<T>(x.getf(2 * p) * r) * w.getf(2 * p);
+    const float b = to_storage<T>(x.getf(2 * p + 1) * r) * w.getf(2 * p + 1);
+    y.setf_pair(p, a, b);
+  }
+  return y;
+}
+
+template <typename T, int kSteps>
+__global__ __launch_bounds__(256)
+void kv_append_norm_rope_kernel(const AppendKernelArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int sub = lane & (kLanesPerRow - 1);            // 8-element slice of a head row
+  const int head_in_step = lane >> 4;                   // 0..3
+  const int tok = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int row = blockIdx.z;
+
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    if (a.global_end) a.global_end[row] = a.new_global[row];
+    if (a.local_end) a.local_end[row] = a.new_local[row];
+  }
+  if (tok >= a.tokens) return;                          // whole waves leave together
+
+  const int fi = tok / a.frame_tokens;
+  const int rem = tok - fi * a.frame_tokens;
+  const int hi = rem / a.grid_w;
+  const int wi = rem - hi * a.grid_w;
+  double2 cs[4];
+  sdv2::load_rotation(a.freqs, a.pairs, a.split_t, a.split_h, sub, a.start_frame[row] + fi, hi, wi, cs);
+
+  const int64_t e0 = sub * 8;
+  const int64_t dst_tok = a.dst_start[row] + tok;
+  const T* qi = static_cast<const T*>(a.q_in) + row * a.q_in_st.row + tok * a.q_in_st.token + e0;
+  const T* ki = static_cast<const T*>(a.k_in) + row * a.k_in_st.row + tok * a.k_in_st.token + e0;
+  const T* vi = static_cast<const T*>(a.v_in) + row * a.v_in_st.row + tok * a.v_in_st.token + e0;
+  T* qo = static_cast<T*>(a.q_out) + row * a.q_out_st.row + tok * a.q_out_st.token + e0;
+  T* kc = static_cast<T*>(a.k_cache) + row * a.k_st.row + dst_tok * a.k_st.token + e0;
+  T* vc = static_cast<T*>(a.v_cache) + row * a.v_st.row + dst_tok * a.v_st.token + e0;
+  const int steps = (a.heads + 3) >> 2;
+
+  sdv2::Vec8<T> q[kSteps], k[kSteps];
+  float ssq_q = 0.f, ssq_k = 0.f;
+#pragma unroll
+  for (int j = 0; j < kSteps; ++j) {
+    const int h = 4 * j + head_in_step;
+    if (j < steps && h < a.heads) {
+      q[j] = sdv2::Vec8<T>::load(qi + h * a.q_in_st.head);
+      k[j] = sdv2::Vec8<T>::load(ki + h * a.k_in_st.head);
+      sdv2::Vec8<T>::load(vi + h * a.v_in_st.head).store(vc + h * a.v_st.head);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        ssq_q += q[j].getf(i) * q[j].getf(i);
+        ssq_k += k[j].getf(i) * k[j].getf(i);
+      }
+    }
+  }
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    ssq_q += __shfl_xor(ssq_q, off, 64);
+    ssq_k += __shfl_xor(ssq_k, off, 64);
+  }
+  const float width = static_cast<float>(a.heads * 128);
+  const float rq = 1.0f / sqrtf(ssq_q / width + a.norm_eps);
+  const float rk = 1.0f / sqrtf(ssq_k / width + a.norm_eps);
+  const T* wq = static_cast<const T*>(a.q_norm_w) + e0;
+  const T* wk = static_cast<const T*>(a.k_norm_w) + e0;
+#pragma unroll
+  for (int j = 0; j < kSteps; ++j) {
+    const int h = 4 * j + head_in_step;
+    if (j < steps && h < a.heads) {
+      const sdv2::Vec8<T> qn = normalise(q[j], rq, sdv2::Vec8<T>::load(wq + h * 128));
+      const sdv2::Vec8<T> kn = normalise(k[j], rk, sdv2::Vec8<T>::load(wk + h * 128));
+      sdv2::rotate(qn, cs).store(qo + h * a.q_out_st.head);
+      sdv2::rotate(kn, cs).store(kc + h * a.k_st.head);
+    }
+  }
+}
+
 bool stride_ok(const sdv2_stride3& s, int vec) {
   return s.row % vec == 0 && s.token % vec == 0 && s.head % vec == 0;
 }
@@ -120,6 +230,14 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
   if ((p->global_end_index || p->local_end_index) && (!p->new_global_end || !p->new_local_end))
     return SDV2_ERR_INVALID_ARG;
   const bool with_q = p->q_in != nullptr;
+  const bool with_norm = p->q_norm_weight != nullptr || p->k_norm_weight != nullptr;
+  if (with_norm) {
+    // the fused norm covers q and k together, as qkv_fn applies it
+    if (!p->q_norm_weight || !p->k_norm_weight || !with_q) return SDV2_ERR_INVALID_ARG;
+    if (p->heads > 4 * kNormMaxSteps) return SDV2_ERR_UNSUPPORTED;
+    if (!(p->norm_eps >= 0.f)) return SDV2_ERR_INVALID_ARG;
+    if (!aligned16(p->q_norm_weight) || !aligned16(p->k_norm_weight)) return SDV2_ERR_INVALID_ARG;
+  }
 
   // 16-byte vector access: 8 bf16 or 4 floats per transaction.
   const int vec = p->dtype == SDV2_BF16 ? 8 : 4;
@@ -144,6 +262,7 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
   a.q_in_st = p->q_in_stride; a.k_in_st = p->k_in_stride; a.v_in_st = p->v_in_stride;
   a.q_out_st = p->q_out_stride; a.k_st = p->k_cache_stride; a.v_st = p->v_cache_stride;
   a.freqs = reinterpret_cast<const double2*>(p->freqs);
+  a.q_norm_w = p->q_norm_weight; a.k_norm_w = p->k_norm_weight; a.norm_eps = p->norm_eps;
   a.global_end = p->global_end_index;
   a.local_end = p->local_end_index;
   a.tokens = p->tokens; a.heads = p->heads; a.grid_w = p->grid_w;
@@ -164,6 +283,22 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
   dim3 grid((p->tokens + kTokensPerBlock - 1) / kTokensPerBlock,
             (p->heads + kHeadsPerThread - 1) / kHeadsPerThread, p->rows);
   hipStream_t stream = static_cast<hipStream_t>(p->stream);
+  if (with_norm) {
+    const dim3 norm_grid((p->tokens + 3) / 4, 1, p->rows);
+    // the q / k slices of a token stay in registers: the variant fixes how many heads / 4 fit
+    auto launch = [&](auto steps_c) {
+      constexpr int kS = decltype(steps_c)::value;
+      if (p->dtype == SDV2_BF16)
+        hipLaunchKernelGGL((kv_append_norm_rope_kernel<uint16_t, kS>), norm_grid, block, 0, stream, a);
+      else
+        hipLaunchKernelGGL((kv_append_norm_rope_kernel<float, kS>), norm_grid, block, 0, stream, a);
+    };
+    const int steps = (p->heads + 3) / 4;
+    if (steps <= 4) launch(std::integral_constant<int, 4>{});
+    else if (steps <= 10) launch(std::integral_constant<int, 10>{});
+    else launch(std::integral_constant<int, kNormMaxSteps>{});
+    return hipGetLastError() == hipSuccess ? SDV2_OK : SDV2_ERR_LAUNCH;
+  }
   if (p->dtype == SDV2_BF16) {
     if (with_q) hipLaunchKernelGGL((kv_append_rope_kernel<uint16_t, true>), grid, block, 0, stream, a);
     else hipLaunchKernelGGL((kv_append_rope_kernel<uint16_t, false>), grid, block, 0, stream, a);

@@ -32,6 +32,14 @@ struct Vec8<uint16_t> {                     // bf16 bit patterns
     (&raw.x)[p] = f32_to_bf16_rne(static_cast<float>(re)) |
                   (f32_to_bf16_rne(static_cast<float>(im)) << 16);
   }
+  __device__ float getf(int i) const {
+    const uint32_t w = (&raw.x)[i >> 1];
+    return __uint_as_float((i & 1) ? (w & 0xffff0000u) : (w << 16));
+  }
+  // element i = x rounded to the storage type (bf16, nearest-even)
+  __device__ void setf_pair(int p, float lo, float hi) {
+    (&raw.x)[p] = f32_to_bf16_rne(lo) | (f32_to_bf16_rne(hi) << 16);
+  }
 };
 
 template <>
@@ -54,6 +62,12 @@ struct Vec8<float> {
     float* dst = p < 2 ? &lo.x + 2 * p : &hi.x + 2 * (p - 2);
     dst[0] = static_cast<float>(re);
     dst[1] = static_cast<float>(im);
+  }
+  __device__ float getf(int i) const { return i < 4 ? (&lo.x)[i] : (&hi.x)[i - 4]; }
+  __device__ void setf_pair(int p, float a, float b) {
+    float* dst = p < 2 ? &lo.x + 2 * p : &hi.x + 2 * (p - 2);
+    dst[0] = a;
+    dst[1] = b;
   }
 };
 

@@ -74,6 +74,15 @@ def device_freqs(freqs: torch.Tensor, device: torch.device) -> torch.Tensor:
     return table
 
 
+def _check_norm(qk_norm, dtype, heads: int, dev) -> None:
+    wq, wk, eps = qk_norm
+    for w in (wq, wk):
+        if w.dtype != dtype or w.numel() != heads * HEAD_DIM or not w.is_contiguous() or w.device != dev:
+            raise RuntimeError(f"norm weights must be contiguous {dtype} tensors of {heads * HEAD_DIM} elements on {dev}")
+    if not eps >= 0:
+        raise RuntimeError("norm eps must be >= 0")
+
+
 def kv_append_rope(
     q: Optional[torch.Tensor],
     k: torch.Tensor,
@@ -89,9 +98,14 @@ def kv_append_rope(
     local_end_index: Optional[torch.Tensor] = None,
     new_global_end: Optional[Sequence[int]] = None,
     new_local_end: Optional[Sequence[int]] = None,
+    qk_norm: Optional[Tuple[torch.Tensor, torch.Tensor, float]] = None,
 ) -> Optional[torch.Tensor]:
     """RoPE q and k, write k' and v into the cache at ``dst_starts`` and store
     the new end indices.  Returns the roped query (``q_out`` or a new tensor).
+
+    ``qk_norm`` = (q weight, k weight, eps) folds the WanRMSNorm of the
+    projection outputs in (wan_base/modules/model.py:70-86): q and k are then
+    the raw projection outputs.
 
     ``freqs_table`` is :func:`device_freqs` output.  Rows are processed in
     groups of at most 16 per launch.
@@ -117,6 +131,10 @@ def kv_append_rope(
             raise RuntimeError("end-index tensors must be contiguous int64 with one entry per row")
     if freqs_table.dtype != torch.float64 or not freqs_table.is_contiguous():
         raise RuntimeError("freqs_table must be the contiguous float64 view from device_freqs()")
+    if qk_norm is not None:
+        _check_norm(qk_norm, k.dtype, heads, dev)
+        if q is None:
+            raise RuntimeError("the fused q/k norm needs q")
 
     lib = _capi.lib()
     stream = _stream_ptr(dev)
@@ -154,6 +172,9 @@ def kv_append_rope(
                 if local_end_index is not None:
                     p.local_end_index = local_end_index.data_ptr() + 8 * r0
             p.stream = stream
+            if qk_norm is not None:
+                p.q_norm_weight, p.k_norm_weight = qk_norm[0].data_ptr(), qk_norm[1].data_ptr()
+                p.norm_eps = float(qk_norm[2])
             _capi.check(lib.sdv2_kv_append_rope(C.byref(p)), "sdv2_kv_append_rope")
     return q_out
 
@@ -331,7 +352,7 @@ class LayerLauncher:
         return (tuple(t.shape), tuple(t.stride()), t.dtype)
 
     def __init__(self, k_cache, v_cache, global_end_index, local_end_index, freqs_table, grid, q_like, k_like=None,
-                 v_like=None):
+                 v_like=None, qk_norm=None):
         k_like = q_like if k_like is None else k_like
         v_like = q_like if v_like is None else v_like
         rows, tokens, heads, _ = q_like.shape
@@ -373,6 +394,11 @@ class LayerLauncher:
         ap.local_end_index = local_end_index.data_ptr()
         ap.new_global_end = C.cast(self.ng, C.POINTER(C.c_int64))
         ap.new_local_end = C.cast(self.nl, C.POINTER(C.c_int64))
+        self.qk_norm = qk_norm
+        if qk_norm is not None:
+            _check_norm(qk_norm, q_like.dtype, heads, dev)
+            ap.q_norm_weight, ap.k_norm_weight = qk_norm[0].data_ptr(), qk_norm[1].data_ptr()
+            ap.norm_eps = float(qk_norm[2])
         self.ap, self.ap_ref = ap, C.byref(ap)
         self.freqs_table = freqs_table
 
@@ -386,8 +412,14 @@ class LayerLauncher:
         self.out_stride = None
         self.forced_splits = 0                       # 0 = the library's own choice
 
-    def matches(self, q, k, v, kv_cache, freqs_table) -> bool:
+    def matches(self, q, k, v, kv_cache, freqs_table, qk_norm=None) -> bool:
         if (self._sig(q), self._sig(k), self._sig(v)) != self.in_sig or freqs_table is not self.freqs_table:
+            return False
+        if (qk_norm is None) != (self.qk_norm is None):
+            return False
+        if qk_norm is not None and (qk_norm[0].data_ptr() != self.qk_norm[0].data_ptr()
+                                    or qk_norm[1].data_ptr() != self.qk_norm[1].data_ptr()
+                                    or float(qk_norm[2]) != float(self.qk_norm[2])):
             return False
         kc, vc = kv_cache["k"], kv_cache["v"]
         return self.cache_sig == (kc.data_ptr(), vc.data_ptr(), tuple(kc.shape), tuple(kc.stride()), tuple(vc.stride()),

@@ -1,0 +1,152 @@
+"""The q / k RMSNorm of the projection outputs (WanRMSNorm,
+wan_base/modules/model.py:70-86; applied in qkv_fn, causal_model.py:212-218)
+folded into the append kernel.
+
+CPU: the oracle's restatement against float64 numpy and the placement of the
+two roundings.  GPU: fused norm + RoPE + append against oracle norm -> oracle
+RoPE.  The sum of squares is an fp32 sum whose order differs between the
+kernel and torch, so the normalised value may differ in its last fp32 bit and
+a stored element by one ulp of the storage type now and then: required here
+are >= 99.99 % identical elements and never more than one ulp (bf16), 2e-6 of
+the largest magnitude (fp32); V and the indices stay exact."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import sdv2_oracle as oracle
+
+
+def test_oracle_rms_norm_against_float64():
+    torch.manual_seed(0)
+    x = torch.randn(2, 5, 256)
+    w = torch.rand(256) + 0.5
+    got = oracle.wan_rms_norm(x, w, 1e-6)
+    xd = x.double().numpy()
+    want = xd / np.sqrt((xd ** 2).mean(-1, keepdims=True) + 1e-6) * w.double().numpy()
+    assert np.allclose(got.numpy(), want, rtol=2e-6, atol=1e-7)
+    # a constant row: x / |x| * w, eps negligible
+    c = torch.full((1, 1, 256), 3.0)
+    assert torch.allclose(oracle.wan_rms_norm(c, w, 0.0), w.view(1, 1, -1), rtol=1e-6)
+    # eps matters for a zero row: no NaN
+    assert torch.equal(oracle.wan_rms_norm(torch.zeros(1, 1, 256), w, 1e-6), torch.zeros(1, 1, 256))
+
+
+def test_oracle_rms_norm_rounds_before_the_weight():
+    """In bf16 the normalised value is rounded to bf16 first and the product
+    with the weight once more (type_as(x) * weight), not once at the end."""
+    torch.manual_seed(1)
+    x = torch.randn(1, 7, 256).bfloat16()
+    w = (torch.rand(256) + 0.5).bfloat16()
+    got = oracle.wan_rms_norm(x, w, 1e-6)
+    xf = x.float()
+    r = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-6)
+    two_roundings = ((xf * r).bfloat16().float() * w.float()).bfloat16()
+    one_rounding = (xf * r * w.float()).bfloat16()
+    assert torch.equal(got, two_roundings)
+    assert not torch.equal(got, one_rounding)
+
+
+def _ulp_diff_bf16(a, b):
+    ia = a.contiguous().view(torch.int16).to(torch.int32)
+    ib = b.contiguous().view(torch.int16).to(torch.int32)
+    # map sign-magnitude to a monotone integer line
+    ia = torch.where(ia < 0, -(ia & 0x7fff), ia)
+    ib = torch.where(ib < 0, -(ib & 0x7fff), ib)
+    return (ia - ib).abs()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("heads", [12, 40, 5])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_fused_norm_append(gpu_device, heads, dtype):
+    from streamdiffusionv2_amd import ops, ring, rope
+
+    print(f"fused q/k norm: heads={heads} {dtype}", flush=True)
+    torch.manual_seed(2)
+    rows, grid, cap = 2, (2, 5, 6), 240
+    S, eps = 60, 1e-6
+    freqs = rope.build_freqs()
+    q = (torch.randn(rows, S, heads, 128) * 1.7).to(dtype)
+    k = (torch.randn(rows, S, heads, 128) * 0.6).to(dtype)
+    v = torch.randn(rows, S, heads, 128).to(dtype)
+    wq = (torch.rand(heads * 128) + 0.5).to(dtype)
+    wk = (torch.rand(heads * 128) + 0.5).to(dtype)
+    start_frames, dst = [3, 9], [60, 120]
+
+    qn = oracle.wan_rms_norm(q.flatten(2), wq, eps).view_as(q)
+    kn = oracle.wan_rms_norm(k.flatten(2), wk, eps).view_as(k)
+    want_q = oracle.causal_rope_apply(qn, [grid] * rows, oracle.build_freqs(), start_frames).type_as(v)
+    want_k = oracle.causal_rope_apply(kn, [grid] * rows, oracle.build_freqs(), start_frames).type_as(v)
+
+    caches = ring.new_kv_cache(1, 1, cap, heads, 1, dtype=dtype, device=gpu_device)
+    ring.replicate_for_stream_batch(caches, rows)
+    cache = caches[0]
+    table = ops.device_freqs(freqs, gpu_device)
+    got_q = ops.kv_append_rope(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), cache["k"], cache["v"], table,
+                               grid, start_frames, dst, global_end_index=cache["global_end_index"],
+                               local_end_index=cache["local_end_index"], new_global_end=[7, 8], new_local_end=[9, 10],
+                               qk_norm=(wq.to(gpu_device), wk.to(gpu_device), eps))
+    torch.cuda.synchronize()
+    got_k = torch.stack([cache["k"][r, dst[r]:dst[r] + S] for r in range(rows)]).cpu()
+    got_v = torch.stack([cache["v"][r, dst[r]:dst[r] + S] for r in range(rows)]).cpu()
+    assert torch.equal(got_v, v)
+    assert cache["global_end_index"].cpu().tolist() == [7, 8] and cache["local_end_index"].cpu().tolist() == [9, 10]
+    for got, want in ((got_q.cpu(), want_q), (got_k, want_k)):
+        if dtype == torch.bfloat16:
+            d = _ulp_diff_bf16(got, want)
+            assert d.max().item() <= 1, d.max().item()
+            assert (d == 0).float().mean().item() >= 0.9999
+        else:
+            # a rotated component is a difference of two products: bound against the vector's scale
+            assert (got - want).abs().max().item() <= 2e-6 * want.abs().max().item()
+    # the untouched part of the cache stays zero
+    assert not cache["k"][0, :dst[0]].any() and not cache["k"][1, dst[1] + S:].any()
+
+
+@pytest.mark.gpu
+def test_module_with_and_without_fusion(gpu_device):
+    from streamdiffusionv2_amd import ring, rope
+    from streamdiffusionv2_amd.attention import CausalWanSelfAttention
+
+    torch.manual_seed(3)
+    dim, heads, grid = 256, 2, (1, 4, 6)
+    S = 24
+    mod = CausalWanSelfAttention(dim, heads).to(gpu_device).bfloat16()
+    with torch.no_grad():
+        mod.norm_q.weight.uniform_(0.5, 1.5)
+        mod.norm_k.weight.uniform_(0.5, 1.5)
+    mod.sink_size = 1
+    freqs = rope.build_freqs()
+    x = [torch.randn(1, S, dim, device=gpu_device).bfloat16() for _ in range(5)]
+    outs = []
+    for fuse in (True, False):
+        mod.fuse_qk_norm = fuse
+        mod.evict_idx = None
+        cache = ring.new_kv_cache(1, 1, 3 * S, heads, 1, device=gpu_device)[0]
+        res = []
+        with torch.no_grad():
+            for c in range(5):
+                res.append(mod(x[c], None, torch.tensor([grid]), freqs, None, kv_cache=cache, current_start=c * S))
+        outs.append((torch.stack(res), cache["k"].clone(), cache["v"].clone()))
+    torch.cuda.synchronize()
+    (y1, k1, v1), (y0, k0, v0) = outs
+    assert torch.equal(v1, v0)
+    d = _ulp_diff_bf16(k1.cpu(), k0.cpu())
+    assert d.max().item() <= 1 and (d == 0).float().mean().item() >= 0.999
+    assert (y1.float() - y0.float()).abs().max().item() <= 3e-2
+
+
+@pytest.mark.gpu
+def test_fused_norm_argument_errors(gpu_device):
+    from streamdiffusionv2_amd import ops, rope
+
+    table = ops.device_freqs(rope.build_freqs(), gpu_device)
+    x = torch.zeros(1, 6, 2, 128, dtype=torch.bfloat16, device=gpu_device)
+    cache = torch.zeros(1, 12, 2, 128, dtype=torch.bfloat16, device=gpu_device)
+    w = torch.ones(256, dtype=torch.bfloat16, device=gpu_device)
+    with pytest.raises(RuntimeError):       # wrong length
+        ops.kv_append_rope(x, x, x, cache, cache.clone(), table, (1, 2, 3), [0], [0], qk_norm=(w[:128], w, 1e-6))
+    with pytest.raises(RuntimeError):       # wrong dtype
+        ops.kv_append_rope(x, x, x, cache, cache.clone(), table, (1, 2, 3), [0], [0], qk_norm=(w.float(), w, 1e-6))
+    with pytest.raises(RuntimeError):       # k only
+        ops.kv_append_rope(None, x, x, cache, cache.clone(), table, (1, 2, 3), [0], [0], qk_norm=(w, w, 1e-6))
