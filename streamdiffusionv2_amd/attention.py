@@ -193,9 +193,10 @@ class CausalWanSelfAttention(nn.Module, RingKVPath):
         self.qk_norm = qk_norm
         self.eps = eps
 
-        # the q / k RMSNorm inside the append kernel (its sum of squares is
-        # taken in another order than torch's, see sdv2_append_params)
-        self.fuse_qk_norm = True
+        # True runs the q / k RMSNorm inside the append kernel.  Off by default:
+        # its sum of squares is taken in another order than torch's, so the
+        # cache can then differ from the unfused path by one ulp in rare elements.
+        self.fuse_qk_norm = False
 
         # ring state, same defaults as causal_model.py:177-179
         self.sink_size = 3
