@@ -117,23 +117,13 @@ void kv_append_rope_kernel(const AppendKernelArgs a) {
 constexpr int kNormMaxSteps = 16;           // heads <= 64
 
 template <typename T>
-__device__ __forceinline__ float to_storage(float x);
-template <>
-__device__ __forceinline__ float to_storage<uint16_t>(float x) {
-  return sdv2::bf16_bits_to_f32(sdv2::f32_to_bf16_rne(x));
-}
-template <>
-__device__ __forceinline__ float to_storage<float>(float x) { return x; }
-
-template <typename T>
 __device__ __forceinline__ sdv2::Vec8<T> normalise(const sdv2::Vec8<T>& x, float r, const sdv2::Vec8<T>& w) {
   sdv2::Vec8<T> y;
+  sdv2::Vec8<T> n;                           // x * r in the storage type
 #pragma unroll
-  for (int p = 0; p < 4; ++p) {
-    const float a = to_storage<T>(x.getf(2 * p) * r) * w.getf(2 * p);
-    const float b = to_storage<T>(x.getf(2 * p + 1) * r) * w.getf(2 * p + 1);
-    y.setf_pair(p, a, b);
-  }
+  for (int p = 0; p < 4; ++p) n.setf_pair(p, x.getf(2 * p) * r, x.getf(2 * p + 1) * r);
+#pragma unroll
+  for (int p = 0; p < 4; ++p) y.setf_pair(p, n.getf(2 * p) * w.getf(2 * p), n.getf(2 * p + 1) * w.getf(2 * p + 1));
   return y;
 }
 

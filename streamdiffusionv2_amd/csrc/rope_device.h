@@ -29,8 +29,7 @@ struct Vec8<uint16_t> {                     // bf16 bit patterns
     return static_cast<double>(__uint_as_float(bits));
   }
   __device__ void set_pair(int p, double re, double im) {
-    (&raw.x)[p] = f32_to_bf16_rne(static_cast<float>(re)) |
-                  (f32_to_bf16_rne(static_cast<float>(im)) << 16);
+    (&raw.x)[p] = pack_bf16_rne(static_cast<float>(re), static_cast<float>(im));
   }
   __device__ float getf(int i) const {
     const uint32_t w = (&raw.x)[i >> 1];
@@ -38,7 +37,7 @@ struct Vec8<uint16_t> {                     // bf16 bit patterns
   }
   // element i = x rounded to the storage type (bf16, nearest-even)
   __device__ void setf_pair(int p, float lo, float hi) {
-    (&raw.x)[p] = f32_to_bf16_rne(lo) | (f32_to_bf16_rne(hi) << 16);
+    (&raw.x)[p] = pack_bf16_rne(lo, hi);
   }
 };
 

@@ -18,6 +18,18 @@ __device__ __forceinline__ uint32_t f32_to_bf16_rne(float f) {
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
 
+// Two floats -> packed bfloat16 pair (lo in the low half), nearest-even: the
+// hardware conversion v_cvt_pk_bf16_f32.  Same bits as f32_to_bf16_rne for every
+// number; a NaN stays a NaN but keeps its sign and payload bits (PyTorch itself
+// encodes a NaN result differently on its scalar, vectorised and GPU paths:
+// 0x7FC0, 0xFFFF, 0x7FFF).
+__device__ __forceinline__ uint32_t pack_bf16_rne(float lo, float hi) {
+  typedef __attribute__((ext_vector_type(2))) float f32x2_t;
+  typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+  const f32x2_t x = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2_t));
+}
+
 }  // namespace sdv2
 
 #endif  // SDV2KV_INTERNAL_H

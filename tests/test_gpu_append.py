@@ -58,3 +58,39 @@ def test_append_matches_oracle_bitwise(gpu_device, dtype, head_major, grid, head
         assert not kc_cpu[r, mask].any() and not vc_cpu[r, mask].any()
     assert g_idx.tolist() == [100 + r for r in range(rows)]
     assert l_idx.tolist() == [200 + r for r in range(rows)]
+
+
+def test_append_special_values(gpu_device):
+    """NaN of either sign, infinities, signed zeros, bf16 subnormals, values
+    near the largest bf16 and round-to-even ties in the inputs: the rotation in
+    double and the rounding to bf16 must still give the CPU result bit for bit
+    wherever that result is a number; where it is a NaN the GPU result is a
+    NaN too (PyTorch's own paths encode a NaN result differently, so there is
+    no one bit pattern to match)."""
+    from streamdiffusionv2_amd import ops
+
+    torch.manual_seed(7)
+    grid, heads = (1, 4, 8), 2
+    S = 32
+    freqs = oracle.build_freqs()
+    q = torch.randn(1, S, heads, 128)
+    k = torch.randn(1, S, heads, 128)
+    specials = torch.tensor([float("nan"), -float("nan"), float("inf"), -float("inf"), 0.0, -0.0,
+                             1e-40, -1e-40, 3.3895e38, 1.00390625, 1.01171875])
+    idx = torch.randperm(S * heads * 128)[:400]
+    k.view(-1)[idx] = specials[torch.arange(400) % len(specials)]
+    q.view(-1)[idx[:50]] = specials[torch.arange(50) % len(specials)]
+    q, k = q.bfloat16(), k.bfloat16()
+    v = torch.randn(1, S, heads, 128).bfloat16()
+    want_q = oracle.causal_rope_apply(q, [grid], freqs, [5])
+    want_k = oracle.causal_rope_apply(k, [grid], freqs, [5])
+    kc = torch.zeros(1, S, heads, 128, dtype=torch.bfloat16, device=gpu_device)
+    vc = torch.zeros_like(kc)
+    got_q = ops.kv_append_rope(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), kc, vc,
+                               ops.device_freqs(freqs, gpu_device), grid, [5], [0])
+    torch.cuda.synchronize()
+    assert torch.isnan(want_k.float()).any() and torch.isinf(want_k.float()).any()
+    for got, want in ((got_q.cpu(), want_q), (kc.cpu(), want_k)):
+        nan = torch.isnan(want.float())
+        assert torch.equal(torch.isnan(got.float()), nan)
+        assert torch.equal(_bits(got)[~nan], _bits(want)[~nan])
