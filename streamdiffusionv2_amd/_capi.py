@@ -117,6 +117,13 @@ def lib() -> C.CDLL:
     global _LIB
     if _LIB is not None:
         return _LIB
+    # The streams and pointers handed to the library come from PyTorch, so both
+    # must sit on ONE HIP runtime: importing torch first makes the library's
+    # libamdhip64 dependency resolve to the copy torch has already loaded.
+    # Loaded the other way round, the process holds two runtimes and every
+    # launch on a torch stream fails.
+    import torch  # noqa: F401
+
     if not LIB_PATH.exists():
         raise ImportError(
             f"{LIB_PATH} is missing: the KV-cache path has no fallback. Build it with "
