@@ -38,6 +38,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <utility>
 
 #include "sdv2kv.h"
@@ -68,6 +69,7 @@ constexpr int kStages = 3;
 constexpr int kLdsBytes = 2 * kStages * kTileBytes;   // 96 KB
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kCuSlots = 256;               // one workgroup per CU
+constexpr int kMaxDevices = 64;
 
 // LDS map: kStages K tile buffers, then kStages V tile buffers.  The DS
 // instructions carry a 16-bit offset, so V fragment addresses are kept
@@ -919,17 +921,20 @@ extern "C" int sdv2_swa_attn_fwd(const sdv2_attn_params* p) {
   if (items > (1 << 28)) return SDV2_ERR_INVALID_ARG;
   dim3 grid((unsigned)(8 * ((items + 7) / 8)));
   if (p->stages != SDV2_STAGE_MERGE) {
-    // 96 KB of LDS is more than the static limit: ask for it once per process.
+    // 96 KB of LDS is more than the static limit: ask for it once per device.
     // The kernel exists twice: the mask inside the chunk costs the plain
     // variant about 2 % even when it is off, so it gets its own code.
-    static const hipError_t lds_attr = [] {
-      const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(swa_attn_fwd_kernel<false>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-      return e != hipSuccess ? e
-                             : hipFuncSetAttribute(reinterpret_cast<const void*>(swa_attn_fwd_kernel<true>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-    }();
-    if (lds_attr != hipSuccess) return SDV2_ERR_LAUNCH;
+    static std::atomic<bool> lds_ready[kMaxDevices];
+    int device = 0;
+    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return SDV2_ERR_LAUNCH;
+    if (!lds_ready[device].load(std::memory_order_acquire)) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(swa_attn_fwd_kernel<false>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess ||
+          hipFuncSetAttribute(reinterpret_cast<const void*>(swa_attn_fwd_kernel<true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess)
+        return SDV2_ERR_LAUNCH;
+      lds_ready[device].store(true, std::memory_order_release);
+    }
     if (a.mask_block_tokens > 0)
       hipLaunchKernelGGL(swa_attn_fwd_kernel<true>, grid, dim3(kThreads), kLdsBytes, stream, a);
     else

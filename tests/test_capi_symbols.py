@@ -96,6 +96,11 @@ def test_cpu_tensors_are_refused():
     from streamdiffusionv2_amd import ops
 
     q = torch.zeros(1, 8, 1, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU only") as err:
+        ops.flash_attn_with_kvcache(q=q, k_cache=q, v_cache=q, cache_seqlens=None)
+    # the reference turns a RuntimeError that names "DeviceType::CUDA" into a silent
+    # SDPA fallback (causal_model.py:359-372): errors of this path must never look like that
+    assert "DeviceType::CUDA" not in str(err.value)
     with pytest.raises(RuntimeError, match="GPU only"):
         ops.swa_attention(q, q, q)
 

@@ -81,6 +81,8 @@ def test_hand_trace_through_both_switches():
     assert entry["local_end_index"].tolist() == [4 * F] * 2 and entry["global_end_index"].tolist() == [8 * F] * 2
     assert entry["current_step"] == entry["total_steps"] == 2
     assert [[x // F for x in q] for q in path.evict_idx] == [[3, 4, 2], [3, 4, 2]]
+    # independent copies per row, as the reference's own test demands (demo/test_online_inference.py:390-404)
+    assert path.evict_idx[0] is not path.evict_idx[1]
     assert pipe.kv_cache_starts == [8 * F] * 2 and pipe.kv_cache_ends == [9 * F] * 2
     assert not pipe.hidden_states.any()
 
