@@ -103,24 +103,19 @@ def gpu_bench(args, w):
     table = ops.device_freqs(freqs, dev)
 
     def timed_layer(path, q, k, v, cache, starts, timers):
-        """Same launches as attend(), with HIP events between the kernels."""
+        """Same launches as attend(), each kernel with its own timing events
+        (recorded in the kernel's dispatch: the kernel's duration itself)."""
         frame_tokens = w.frame_tokens
         plan = ring.plan_append(cache, path.evict_idx, starts, S, frame_tokens, path.sink_size)
         launcher = path._layer_launcher(q, k, v, cache, table, w.grid)
         launcher.patch(q, k, v, [c // frame_tokens for c in starts], plan, None)
-        ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
-        ev[0].record()
+        split = launcher.at.num_splits > 1
+        t = (ops.KernelTimer(), ops.KernelTimer(), ops.KernelTimer() if split else None)
+        launcher.set_timers(*t)
         launcher.run_append()
-        ev[1].record()
-        if launcher.at.num_splits > 1:
-            launcher.run_attention(_capi.STAGE_PARTIAL)
-            ev[2].record()
-            launcher.run_attention(_capi.STAGE_MERGE)
-        else:
-            launcher.run_attention()
-            ev[2].record()
-        ev[3].record()
-        timers.append(ev)
+        launcher.run_attention()
+        launcher.set_timers()
+        timers.append(t)
 
     # Fast-forward to the steady state without launching anything: the host
     # planner walks through the fill phase (so the eviction queues and indices
@@ -164,9 +159,13 @@ def gpu_bench(args, w):
     for _ in range(args.steps):
         step(timers)
     torch.cuda.synchronize()
-    t_append = sum(e[0].elapsed_time(e[1]) for e in timers) / len(timers)
-    t_attn = sum(e[1].elapsed_time(e[2]) for e in timers) / len(timers)
-    t_merge = sum(e[2].elapsed_time(e[3]) for e in timers) / len(timers)
+    t_append = sum(t[0].elapsed_ms() for t in timers) / len(timers)
+    t_attn = sum(t[1].elapsed_ms() for t in timers) / len(timers)
+    t_merge = sum(t[2].elapsed_ms() for t in timers if t[2]) / len(timers)
+    for t in timers:
+        for x in t:
+            if x:
+                x.close()
     splits = args.num_splits or _capi.lib().sdv2_swa_attn_default_splits(B, S, H, w.cache_tokens)
     fill_ms = None
     if args.fill_phase:

@@ -30,7 +30,7 @@
 extern "C" {
 #endif
 
-#define SDV2KV_ABI_VERSION 2
+#define SDV2KV_ABI_VERSION 3
 #define SDV2_HEAD_DIM 128      /* causal_stream_inference.py:99-100 fixes 128 */
 #define SDV2_MAX_ROWS 16       /* rows (B) per sdv2_kv_append_rope call       */
 #define SDV2_MAX_SINK_FRAMES 16 /* sink frames per sdv2_sink_similarity call  */
@@ -119,6 +119,8 @@ typedef struct sdv2_append_params {
   const void* q_norm_weight;   /* device, or NULL (together with k_norm_weight) */
   const void* k_norm_weight;
   float norm_eps;
+  void* timing_start;          /* optional sdv2 timing events (see sdv2_event_create): */
+  void* timing_stop;           /* recorded with the kernel's own dispatch              */
 } sdv2_append_params;
 
 int sdv2_kv_append_rope(const sdv2_append_params* p);
@@ -169,6 +171,10 @@ typedef struct sdv2_attn_params {
    * [chunk_key_start[i] + (t / b + 1) * b, chunk_key_start[i] + S); everything
    * else in the cache is older and stays visible.  0 (or b >= S) = no mask.  */
   int32_t mask_block_tokens;
+  void* timing_start;          /* optional timing events around the attention kernel   */
+  void* timing_stop;
+  void* merge_timing_start;    /* ... and around the merge kernel of a split call      */
+  void* merge_timing_stop;
   const int32_t* chunk_key_start;  /* device int32 [B], each in [0, L - S]; may be */
                                    /* NULL when the mask is off                    */
 } sdv2_attn_params;
@@ -221,6 +227,19 @@ typedef struct sdv2_sink_sim_params {
 
 size_t sdv2_sink_similarity_workspace_bytes(int32_t rows, int32_t heads, int32_t sink_frames);
 int sdv2_sink_similarity(const sdv2_sink_sim_params* p);
+
+/* ------------------------------------------------------------------------
+ * Timing events.  No counterpart in the reference: they exist for
+ * measurement.  An event handed to a launch through timing_start /
+ * timing_stop is recorded in the dispatch of that one kernel (start when the
+ * kernel begins to execute, stop when it has finished), so the interval is
+ * the kernel's own duration as a profiler reports it, without the gap that
+ * separate event records on the stream would add.  sdv2_event_elapsed_ms
+ * waits for the stop event.
+ * ---------------------------------------------------------------------- */
+int sdv2_event_create(void** event);
+int sdv2_event_destroy(void* event);
+int sdv2_event_elapsed_ms(void* start, void* stop, float* ms);
 
 /* ------------------------------------------------------------------------
  * Plain device-to-device copy of `bytes` bytes with the library's own 16-byte

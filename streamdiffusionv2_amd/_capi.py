@@ -11,7 +11,7 @@ from typing import Optional
 
 LIB_PATH = Path(__file__).resolve().parent / "_lib" / "libsdv2kv.so"
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 HEAD_DIM = 128
 MAX_ROWS = 16
 
@@ -37,6 +37,9 @@ EXPORTED_SYMBOLS = (
     "sdv2_swa_attn_fwd",
     "sdv2_sink_similarity_workspace_bytes",
     "sdv2_sink_similarity",
+    "sdv2_event_create",
+    "sdv2_event_destroy",
+    "sdv2_event_elapsed_ms",
     "sdv2_copy_bytes",
 )
 
@@ -67,6 +70,8 @@ class AppendParams(C.Structure):
         ("q_norm_weight", C.c_void_p),
         ("k_norm_weight", C.c_void_p),
         ("norm_eps", C.c_float),
+        ("timing_start", C.c_void_p),
+        ("timing_stop", C.c_void_p),
     ]
 
 
@@ -84,6 +89,10 @@ class AttnParams(C.Structure):
         ("workspace_bytes", C.c_size_t),
         ("stream", C.c_void_p),
         ("mask_block_tokens", C.c_int32),
+        ("timing_start", C.c_void_p),
+        ("timing_stop", C.c_void_p),
+        ("merge_timing_start", C.c_void_p),
+        ("merge_timing_stop", C.c_void_p),
         ("chunk_key_start", C.c_void_p),
     ]
 
@@ -146,6 +155,12 @@ def lib() -> C.CDLL:
     handle.sdv2_sink_similarity_workspace_bytes.argtypes = [C.c_int32] * 3
     handle.sdv2_sink_similarity.restype = C.c_int
     handle.sdv2_sink_similarity.argtypes = [C.POINTER(SinkSimParams)]
+    handle.sdv2_event_create.restype = C.c_int
+    handle.sdv2_event_create.argtypes = [C.POINTER(C.c_void_p)]
+    handle.sdv2_event_destroy.restype = C.c_int
+    handle.sdv2_event_destroy.argtypes = [C.c_void_p]
+    handle.sdv2_event_elapsed_ms.restype = C.c_int
+    handle.sdv2_event_elapsed_ms.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]
     handle.sdv2_copy_bytes.restype = C.c_int
     handle.sdv2_copy_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
     if handle.sdv2_abi_version() != ABI_VERSION:

@@ -220,6 +220,7 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
   if ((p->global_end_index || p->local_end_index) && (!p->new_global_end || !p->new_local_end))
     return SDV2_ERR_INVALID_ARG;
   const bool with_q = p->q_in != nullptr;
+  if ((p->timing_start == nullptr) != (p->timing_stop == nullptr)) return SDV2_ERR_INVALID_ARG;
   const bool with_norm = p->q_norm_weight != nullptr || p->k_norm_weight != nullptr;
   if (with_norm) {
     // the fused norm covers q and k together, as qkv_fn applies it
@@ -279,9 +280,11 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
     auto launch = [&](auto steps_c) {
       constexpr int kS = decltype(steps_c)::value;
       if (p->dtype == SDV2_BF16)
-        hipLaunchKernelGGL((kv_append_norm_rope_kernel<uint16_t, kS>), norm_grid, block, 0, stream, a);
+        sdv2::launch_timed(kv_append_norm_rope_kernel<uint16_t, kS>, norm_grid, block, 0, stream, p->timing_start,
+                           p->timing_stop, a);
       else
-        hipLaunchKernelGGL((kv_append_norm_rope_kernel<float, kS>), norm_grid, block, 0, stream, a);
+        sdv2::launch_timed(kv_append_norm_rope_kernel<float, kS>, norm_grid, block, 0, stream, p->timing_start,
+                           p->timing_stop, a);
     };
     const int steps = (p->heads + 3) / 4;
     if (steps <= 4) launch(std::integral_constant<int, 4>{});
@@ -290,11 +293,11 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
     return hipGetLastError() == hipSuccess ? SDV2_OK : SDV2_ERR_LAUNCH;
   }
   if (p->dtype == SDV2_BF16) {
-    if (with_q) hipLaunchKernelGGL((kv_append_rope_kernel<uint16_t, true>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((kv_append_rope_kernel<uint16_t, false>), grid, block, 0, stream, a);
+    if (with_q) sdv2::launch_timed(kv_append_rope_kernel<uint16_t, true>, grid, block, 0, stream, p->timing_start, p->timing_stop, a);
+    else sdv2::launch_timed(kv_append_rope_kernel<uint16_t, false>, grid, block, 0, stream, p->timing_start, p->timing_stop, a);
   } else {
-    if (with_q) hipLaunchKernelGGL((kv_append_rope_kernel<float, true>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((kv_append_rope_kernel<float, false>), grid, block, 0, stream, a);
+    if (with_q) sdv2::launch_timed(kv_append_rope_kernel<float, true>, grid, block, 0, stream, p->timing_start, p->timing_stop, a);
+    else sdv2::launch_timed(kv_append_rope_kernel<float, false>, grid, block, 0, stream, p->timing_start, p->timing_stop, a);
   }
   return hipGetLastError() == hipSuccess ? SDV2_OK : SDV2_ERR_LAUNCH;
 }

@@ -1,5 +1,5 @@
 // Small entry points of the sdv2kv C ABI that are not kernels of the path
-// itself: version, status strings and the counter-calibration copy.
+// itself: version, status strings, timing events and the counter-calibration copy.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -26,6 +26,27 @@ extern "C" const char* sdv2_status_string(int status) {
     case SDV2_ERR_LAUNCH: return "kernel launch failed";
     default: return "unknown status";
   }
+}
+
+extern "C" int sdv2_event_create(void** event) {
+  if (!event) return SDV2_ERR_INVALID_ARG;
+  hipEvent_t e = nullptr;
+  if (hipEventCreate(&e) != hipSuccess) return SDV2_ERR_LAUNCH;
+  *event = e;
+  return SDV2_OK;
+}
+
+extern "C" int sdv2_event_destroy(void* event) {
+  if (!event) return SDV2_OK;
+  return hipEventDestroy(static_cast<hipEvent_t>(event)) == hipSuccess ? SDV2_OK : SDV2_ERR_INVALID_ARG;
+}
+
+extern "C" int sdv2_event_elapsed_ms(void* start, void* stop, float* ms) {
+  if (!start || !stop || !ms) return SDV2_ERR_INVALID_ARG;
+  if (hipEventSynchronize(static_cast<hipEvent_t>(stop)) != hipSuccess) return SDV2_ERR_LAUNCH;
+  return hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)) == hipSuccess
+             ? SDV2_OK
+             : SDV2_ERR_INVALID_ARG;
 }
 
 extern "C" int sdv2_copy_bytes(void* dst, const void* src, size_t bytes, void* stream) {

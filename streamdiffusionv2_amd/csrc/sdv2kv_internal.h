@@ -3,9 +3,22 @@
 #define SDV2KV_INTERNAL_H
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 namespace sdv2 {
+
+// Launch with the caller's optional timing events attached to the kernel's own
+// dispatch (both or none).
+template <typename Kernel, typename Args>
+inline void launch_timed(Kernel kernel, dim3 grid, dim3 block, uint32_t lds_bytes, hipStream_t stream, void* start,
+                         void* stop, const Args& args) {
+  if (start && stop)
+    hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, static_cast<hipEvent_t>(start),
+                          static_cast<hipEvent_t>(stop), 0, args);
+  else
+    hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, args);
+}
 
 // float -> bfloat16 bit pattern, round-to-nearest-even, NaN -> 0x7FC0: the
 // rounding PyTorch applies when a float (or a double already narrowed to

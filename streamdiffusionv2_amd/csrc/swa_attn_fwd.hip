@@ -899,6 +899,9 @@ extern "C" int sdv2_swa_attn_fwd(const sdv2_attn_params* p) {
   const float scale = p->softmax_scale > 0.f ? p->softmax_scale : 0.08838834764831845f;  // 1/sqrt(128)
   a.scale_log2 = scale * kLog2e;
   if (p->mask_block_tokens < 0) return SDV2_ERR_INVALID_ARG;
+  if ((p->timing_start == nullptr) != (p->timing_stop == nullptr) ||
+      (p->merge_timing_start == nullptr) != (p->merge_timing_stop == nullptr))
+    return SDV2_ERR_INVALID_ARG;
   if (p->mask_block_tokens > 0 && p->mask_block_tokens < p->q_tokens) {
     // a block as long as the chunk hides nothing: only shorter blocks switch the mask on
     if (!p->chunk_key_start) return SDV2_ERR_INVALID_ARG;
@@ -936,14 +939,17 @@ extern "C" int sdv2_swa_attn_fwd(const sdv2_attn_params* p) {
       lds_ready[device].store(true, std::memory_order_release);
     }
     if (a.mask_block_tokens > 0)
-      hipLaunchKernelGGL(swa_attn_fwd_kernel<true>, grid, dim3(kThreads), kLdsBytes, stream, a);
+      sdv2::launch_timed(swa_attn_fwd_kernel<true>, grid, dim3(kThreads), kLdsBytes, stream, p->timing_start,
+                         p->timing_stop, a);
     else
-      hipLaunchKernelGGL(swa_attn_fwd_kernel<false>, grid, dim3(kThreads), kLdsBytes, stream, a);
+      sdv2::launch_timed(swa_attn_fwd_kernel<false>, grid, dim3(kThreads), kLdsBytes, stream, p->timing_start,
+                         p->timing_stop, a);
     if (hipGetLastError() != hipSuccess) return SDV2_ERR_LAUNCH;
   }
   if (splits > 1 && p->stages != SDV2_STAGE_PARTIAL) {
     const int64_t nq = (int64_t)p->rows * p->heads * p->q_tokens;
-    hipLaunchKernelGGL(swa_attn_merge_kernel, dim3((unsigned)((nq + 15) / 16)), dim3(256), 0, stream, a);
+    sdv2::launch_timed(swa_attn_merge_kernel, dim3((unsigned)((nq + 15) / 16)), dim3(256), 0, stream,
+                       p->merge_timing_start, p->merge_timing_stop, a);
     if (hipGetLastError() != hipSuccess) return SDV2_ERR_LAUNCH;
   }
   return SDV2_OK;

@@ -337,6 +337,37 @@ def sink_similarity(
     return similarity, refresh
 
 
+class KernelTimer:
+    """A start/stop pair of the library's timing events.  Handed to a launch
+    (``LayerLauncher.set_timers``) it is recorded in that kernel's own
+    dispatch, so :meth:`elapsed_ms` is the kernel's duration as a profiler
+    reports it, without the gap separate stream events add."""
+
+    def __init__(self):
+        lib = _capi.lib()
+        self.start, self.stop = C.c_void_p(), C.c_void_p()
+        _capi.check(lib.sdv2_event_create(C.byref(self.start)), "sdv2_event_create")
+        _capi.check(lib.sdv2_event_create(C.byref(self.stop)), "sdv2_event_create")
+
+    def elapsed_ms(self) -> float:
+        ms = C.c_float()
+        _capi.check(_capi.lib().sdv2_event_elapsed_ms(self.start, self.stop, C.byref(ms)), "sdv2_event_elapsed_ms")
+        return ms.value
+
+    def close(self) -> None:
+        lib = _capi.lib()
+        for e in (self.start, self.stop):
+            if e:
+                lib.sdv2_event_destroy(e)
+        self.start, self.stop = C.c_void_p(), C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
 class LayerLauncher:
     """Pre-built launch descriptors for one layer's (append, attention) pair.
 
@@ -463,6 +494,13 @@ class LayerLauncher:
         at.seq_lens = seq_lens.data_ptr() if seq_lens is not None else None
         at.stream = stream
         return out
+
+    def set_timers(self, append: Optional[KernelTimer] = None, attention: Optional[KernelTimer] = None,
+                   merge: Optional[KernelTimer] = None) -> None:
+        """Attach (or, with None, detach) kernel timers for the next launches."""
+        self.ap.timing_start, self.ap.timing_stop = (append.start, append.stop) if append else (None, None)
+        self.at.timing_start, self.at.timing_stop = (attention.start, attention.stop) if attention else (None, None)
+        self.at.merge_timing_start, self.at.merge_timing_stop = (merge.start, merge.stop) if merge else (None, None)
 
     def run_append(self) -> None:
         _capi.check(self.lib.sdv2_kv_append_rope(self.ap_ref), "sdv2_kv_append_rope")
