@@ -122,3 +122,40 @@ def test_c3_full_size(gpu_device):
 def test_c5_full_size_with_outliers(gpu_device):
     w = workloads.WORKLOADS[5]
     _run(w, gpu_device, layers=1, calls=9, sample_rows=24, full_compare_at={0, 7, 8})
+
+
+def test_kernel_timers_measure_each_kernel(gpu_device):
+    """Timing events handed to a launch are recorded with that kernel alone:
+    three positive, plausible durations for append, attention and merge of one
+    layer call, and the call's result is unchanged by them."""
+    from streamdiffusionv2_amd import ops, ring, rope
+    from streamdiffusionv2_amd.attention import RingKVPath
+
+    torch.manual_seed(0)
+    heads, grid, S, cap = 2, (1, 8, 16), 128, 1024
+    freqs = rope.build_freqs()
+    table = ops.device_freqs(freqs, gpu_device)
+    cache = ring.new_kv_cache(1, 1, cap, heads, 1, device=gpu_device)[0]
+    cache["k"].normal_()
+    cache["v"].normal_()
+    path = RingKVPath(sink_size=1)
+    path.num_splits = 2
+    q, k, v = (torch.randn(1, S, heads, 128, device=gpu_device).bfloat16() for _ in range(3))
+    ref = path.attend(q, k, v, torch.tensor([grid]), freqs, cache, [0]).clone()      # builds the launcher
+    path.evict_idx = None
+    cache["global_end_index"].zero_()
+    cache["local_end_index"].zero_()
+    plan = ring.plan_append(cache, [[]], [0], S, 128, 1)
+    launcher = path._layer_launcher(q, k, v, cache, table, grid)
+    out = launcher.patch(q, k, v, [0], plan, None)
+    timers = [ops.KernelTimer() for _ in range(3)]
+    launcher.set_timers(*timers)
+    launcher.run_append()
+    launcher.run_attention()
+    launcher.set_timers()
+    torch.cuda.synchronize()
+    times = [t.elapsed_ms() for t in timers]
+    assert all(0.0 < t < 5.0 for t in times), times
+    assert torch.equal(out, ref)
+    for t in timers:
+        t.close()
