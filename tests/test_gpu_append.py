@@ -94,3 +94,61 @@ def test_append_special_values(gpu_device):
         nan = torch.isnan(want.float())
         assert torch.equal(torch.isnan(got.float()), nan)
         assert torch.equal(_bits(got)[~nan], _bits(want)[~nan])
+
+
+def test_append_random_shapes(gpu_device):
+    """Seeded sweep: grids with 1-4 frames, odd heights / widths, 1-41 heads,
+    1-3 rows, both dtypes, both cache layouts, with and without q, with and
+    without the index stores: cache slot and roped query bit for bit."""
+    from streamdiffusionv2_amd import ops
+
+    rng = torch.Generator().manual_seed(77)
+
+    def ri(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=rng).item())
+
+    freqs = oracle.build_freqs()
+    table = ops.device_freqs(freqs, gpu_device)
+    for case in range(24):
+        grid = (ri(1, 4), ri(1, 9), ri(1, 11))
+        S = grid[0] * grid[1] * grid[2]
+        heads, rows = ri(1, 41) if case % 3 == 0 else ri(1, 6), ri(1, 3)
+        dtype = torch.float32 if case % 4 == 0 else torch.bfloat16
+        head_major, with_q, with_idx = bool(case % 2), case % 5 != 0, case % 3 != 1
+        cap = S * ri(1, 3) + ri(0, 7)
+        start_frames = [ri(0, 1024 - grid[0]) for _ in range(rows)]
+        dst = [ri(0, cap - S) for _ in range(rows)]
+        print(f"case {case}: grid={grid} heads={heads} rows={rows} {dtype} head_major={head_major} "
+              f"with_q={with_q} with_idx={with_idx} cap={cap} frames={start_frames} dst={dst}", flush=True)
+        q = torch.randn(rows, S, heads, 128, generator=rng).to(dtype)
+        k = torch.randn(rows, S, heads, 128, generator=rng).to(dtype)
+        v = torch.randn(rows, S, heads, 128, generator=rng).to(dtype)
+        want_q = oracle.causal_rope_apply(q, [grid] * rows, freqs, start_frames)
+        want_k = oracle.causal_rope_apply(k, [grid] * rows, freqs, start_frames)
+        shape = (rows, heads, cap, 128) if head_major else (rows, cap, heads, 128)
+        kc = torch.zeros(shape, dtype=dtype, device=gpu_device)
+        vc = torch.zeros(shape, dtype=dtype, device=gpu_device)
+        if head_major:
+            kc, vc = kc.permute(0, 2, 1, 3), vc.permute(0, 2, 1, 3)
+        g_idx = torch.full((rows,), -1, dtype=torch.long, device=gpu_device)
+        l_idx = torch.full((rows,), -1, dtype=torch.long, device=gpu_device)
+        idx = dict(global_end_index=g_idx, local_end_index=l_idx, new_global_end=list(range(5, 5 + rows)),
+                   new_local_end=list(range(9, 9 + rows))) if with_idx else {}
+        got_q = ops.kv_append_rope(q.to(gpu_device) if with_q else None, k.to(gpu_device), v.to(gpu_device), kc, vc,
+                                   table, grid, start_frames, dst, **idx)
+        torch.cuda.synchronize()
+        if with_q:
+            assert torch.equal(_bits(got_q.cpu()), _bits(want_q)), case
+        else:
+            assert got_q is None
+        kc_cpu, vc_cpu = kc.cpu(), vc.cpu()
+        for r in range(rows):
+            assert torch.equal(_bits(kc_cpu[r, dst[r]:dst[r] + S]), _bits(want_k[r])), (case, r)
+            assert torch.equal(_bits(vc_cpu[r, dst[r]:dst[r] + S]), _bits(v[r])), (case, r)
+            outside = torch.ones(cap, dtype=torch.bool)
+            outside[dst[r]:dst[r] + S] = False
+            assert not kc_cpu[r, outside].any() and not vc_cpu[r, outside].any(), (case, r)
+        if with_idx:
+            assert g_idx.tolist() == list(range(5, 5 + rows)) and l_idx.tolist() == list(range(9, 9 + rows))
+        else:
+            assert g_idx.tolist() == [-1] * rows

@@ -91,3 +91,43 @@ def test_attention_tiny_sequences(gpu_device):
         got = ops.swa_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), None)
         torch.cuda.synchronize()
         _check(got.cpu(), want)
+
+
+def test_attention_random_shapes(gpu_device):
+    """Seeded sweep over small shapes: odd token counts, single keys, more
+    splits than tiles, per-row lengths including 1, both cache layouts, head
+    counts 1-5, optional mask inside the chunk.  Every case against the fp32
+    oracle."""
+    from streamdiffusionv2_amd import ops
+
+    rng = torch.Generator().manual_seed(2024)
+
+    def ri(lo, hi):
+        return int(torch.randint(lo, hi + 1, (1,), generator=rng).item())
+
+    for case in range(48):
+        rows, heads = ri(1, 3), ri(1, 5)
+        S = ri(1, 520) if case % 3 else ri(1, 40)
+        L = max(S, ri(1, 1400)) if case % 2 else ri(1, 1400)
+        splits = [0, 1, 2, 3, 5, 9][ri(0, 5)]
+        lens = [ri(1, L) for _ in range(rows)] if case % 4 == 0 else [L] * rows
+        head_major = bool(case % 2)
+        masked = L >= S and S >= 2 and case % 5 == 0 and lens == [L] * rows
+        bt = ri(1, S - 1) if masked else 0
+        starts = [ri(0, L - S) for _ in range(rows)] if masked else None
+        print(f"case {case}: rows={rows} heads={heads} S={S} L={L} splits={splits} lens={lens} "
+              f"head_major={head_major} bt={bt} starts={starts}", flush=True)
+        q = torch.randn(rows, S, heads, 128, generator=rng).bfloat16()
+        k = torch.randn(rows, L, heads, 128, generator=rng).bfloat16()
+        v = torch.randn(rows, L, heads, 128, generator=rng).bfloat16()
+        want = oracle.attention_fp32_reference(q, k, v, lens, starts, bt)
+        if head_major:
+            kd = k.permute(0, 2, 1, 3).contiguous().to(gpu_device).permute(0, 2, 1, 3)
+            vd = v.permute(0, 2, 1, 3).contiguous().to(gpu_device).permute(0, 2, 1, 3)
+        else:
+            kd, vd = k.to(gpu_device), v.to(gpu_device)
+        sl = torch.tensor(lens, dtype=torch.int32, device=gpu_device) if lens != [L] * rows else None
+        kw = dict(chunk_key_start=starts, mask_block_tokens=bt) if masked else {}
+        got = ops.swa_attention(q.to(gpu_device), kd, vd, sl, num_splits=splits, **kw)
+        torch.cuda.synchronize()
+        _check(got.cpu(), want)
