@@ -159,3 +159,54 @@ def test_kernel_timers_measure_each_kernel(gpu_device):
     assert torch.equal(out, ref)
     for t in timers:
         t.close()
+
+
+def test_layer_call_replays_from_a_hip_graph(gpu_device):
+    """The library neither allocates nor synchronises, so a layer call (append,
+    split attention, merge) can be captured into a HIP graph.  A captured call
+    always writes the slot it was planned for, so it is replayed here for that
+    slot with fresh inputs in the same static buffers; every replay, with eager
+    work and synchronisations in between, must equal the eager result."""
+    from streamdiffusionv2_amd import ops, ring, rope
+
+    torch.manual_seed(1)
+    heads, grid, S, cap = 2, (1, 8, 16), 128, 1024
+    table = ops.device_freqs(rope.build_freqs(), gpu_device)
+    cache = ring.new_kv_cache(1, 1, cap, heads, 1, device=gpu_device)[0]
+    cache["k"].normal_()
+    cache["v"].normal_()
+    cache["local_end_index"].fill_(cap)
+    cache["global_end_index"].fill_(10 * S)
+    base_k, base_v = cache["k"].clone(), cache["v"].clone()
+    q, k, v = (torch.zeros(1, S, heads, 128, device=gpu_device, dtype=torch.bfloat16) for _ in range(3))
+    plan = ring.AppendPlan([3 * S], [11 * S], [cap])
+    launcher = ops.LayerLauncher(cache["k"], cache["v"], cache["global_end_index"], cache["local_end_index"],
+                                 table, grid, q)
+    launcher.forced_splits = 2
+    ops._workspace(gpu_device, 1 << 22)            # grown before the capture, not inside it
+
+    def call():
+        return launcher.launch(q, k, v, [10], plan, None)
+
+    call()                                         # warm-up outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_static = call()
+    for trial in range(4):
+        fresh = [torch.randn(1, S, heads, 128, device=gpu_device).bfloat16() for _ in range(3)]
+        for dst, src in zip((q, k, v), fresh):
+            dst.copy_(src)
+        cache["k"].copy_(base_k)
+        cache["v"].copy_(base_v)
+        graph.replay()
+        torch.cuda.synchronize()
+        got, got_k = out_static.clone(), cache["k"].clone()
+        # the same call eagerly, from the same starting cache
+        cache["k"].copy_(base_k)
+        cache["v"].copy_(base_v)
+        want = call().clone()
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), trial
+        assert torch.equal(got_k, cache["k"]), trial
+        assert cache["global_end_index"].tolist() == [11 * S]
