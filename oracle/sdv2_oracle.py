@@ -23,10 +23,18 @@ replicate_for_stream_batch models/wan/causal_stream_inference.py:221-225
 StreamShiftRegister        models/wan/causal_stream_inference.py:248-272
 chunk_schedule             streamdiffusionv2/pipeline.py:235-279, 386-391
 noise_scale_and_step       streamv2v/inference.py:51-57
+wan_rms_norm               models/wan/wan_base/modules/model.py:70-86
+chunk_block_mask           models/wan/causal_model.py:670-686 (carried over to
+                           cache positions)
+cross_attention_with_cache models/wan/wan_base/modules/model.py:160-196
+new_crossattn_cache        models/wan/causal_stream_inference.py:109-122
 =========================  ====================================================
 
 Pinning (what fixes each function independently of this file) lives in
-``tests/test_oracle_*.py``: closed forms for the tables, a scalar IEEE-double
+``tests/test_oracle_*.py`` (and, for the four functions at the end of the
+table, in ``tests/test_fused_qk_norm.py``, ``tests/test_block_mask.py``,
+``tests/test_cross_attention_cache.py``; the adaptive sink refresh inside
+``RingAttentionOracle.step`` in ``tests/test_oracle_adaptive_sink.py``): closed forms for the tables, a scalar IEEE-double
 loop for the rotation and its double->float->bf16 rounding, hand traces of the
 slot schedule held as JSON under ``tests/golden/``, brute-force list
 simulation of the ring, and a float64 numpy softmax for the attention.  The
