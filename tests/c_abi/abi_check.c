@@ -1,0 +1,63 @@
+/* A plain C caller of the sdv2kv C ABI: proves that include/sdv2kv.h is C
+ * (not C++), that the library links from C, and that argument validation
+ * answers with status codes before anything touches a GPU.  Built and run by
+ * tests/test_capi_symbols.py; prints one line per check. */
+#include <stdio.h>
+#include <string.h>
+
+#include "sdv2kv.h"
+
+static int failures = 0;
+
+static void expect(const char* what, int got, int want) {
+  printf("%s: %d (%s)%s\n", what, got, sdv2_status_string(got), got == want ? "" : "  <-- UNEXPECTED");
+  if (got != want) ++failures;
+}
+
+int main(void) {
+  if (sdv2_abi_version() != SDV2KV_ABI_VERSION) {
+    printf("ABI version %d, header says %d\n", sdv2_abi_version(), SDV2KV_ABI_VERSION);
+    return 2;
+  }
+  expect("append(NULL)", sdv2_kv_append_rope(NULL), SDV2_ERR_INVALID_ARG);
+  expect("attention(NULL)", sdv2_swa_attn_fwd(NULL), SDV2_ERR_INVALID_ARG);
+  expect("sink_similarity(NULL)", sdv2_sink_similarity(NULL), SDV2_ERR_INVALID_ARG);
+
+  sdv2_append_params ap;
+  memset(&ap, 0, sizeof ap);
+  ap.head_dim = 64;
+  expect("append head_dim 64", sdv2_kv_append_rope(&ap), SDV2_ERR_UNSUPPORTED);
+  ap.head_dim = SDV2_HEAD_DIM;
+  ap.dtype = 7;
+  expect("append unknown dtype", sdv2_kv_append_rope(&ap), SDV2_ERR_UNSUPPORTED);
+  ap.dtype = SDV2_BF16;
+  ap.heads = 12;
+  ap.rows = SDV2_MAX_ROWS + 1;
+  expect("append too many rows", sdv2_kv_append_rope(&ap), SDV2_ERR_INVALID_ARG);
+  ap.rows = 0;
+  expect("append of nothing", sdv2_kv_append_rope(&ap), SDV2_OK);
+  ap.rows = 1;
+  ap.tokens = 6;
+  ap.grid_f = 1; ap.grid_h = 2; ap.grid_w = 2;     /* 4 != 6 tokens */
+  expect("append grid/tokens mismatch", sdv2_kv_append_rope(&ap), SDV2_ERR_INVALID_ARG);
+
+  sdv2_attn_params at;
+  memset(&at, 0, sizeof at);
+  at.head_dim = 96;
+  expect("attention head_dim 96", sdv2_swa_attn_fwd(&at), SDV2_ERR_UNSUPPORTED);
+  at.head_dim = SDV2_HEAD_DIM;
+  at.heads = 12;
+  at.rows = 0;
+  expect("attention of nothing", sdv2_swa_attn_fwd(&at), SDV2_OK);
+  at.rows = 1; at.q_tokens = 8; at.max_seq_len = 8;
+  expect("attention null tensors", sdv2_swa_attn_fwd(&at), SDV2_ERR_INVALID_ARG);
+
+  printf("splits for 1x1560 tokens, 12 heads, 9360 keys: %d\n", sdv2_swa_attn_default_splits(1, 1560, 12, 9360));
+  printf("workspace for that call: %zu bytes\n", sdv2_swa_attn_workspace_bytes(1, 1560, 12, 9360, 0));
+  printf("sink-similarity workspace, 1 row, 12 heads, 3 sink frames: %zu bytes\n",
+         sdv2_sink_similarity_workspace_bytes(1, 12, 3));
+  expect("event_create(NULL)", sdv2_event_create(NULL), SDV2_ERR_INVALID_ARG);
+  expect("copy of nothing", sdv2_copy_bytes(NULL, NULL, 0, NULL), SDV2_OK);
+  printf(failures ? "FAILED: %d\n" : "all checks passed\n", failures);
+  return failures ? 1 : 0;
+}

@@ -119,3 +119,30 @@ def test_module_signature_matches_reference():
     assert {n for n, _ in m.named_children()} == {"q", "k", "v", "o", "norm_q", "norm_k"}
     with pytest.raises(NotImplementedError):
         m(torch.zeros(1, 4, 256), None, None, None, None, kv_cache=None)
+
+
+def test_plain_c_caller(tmp_path):
+    """include/sdv2kv.h compiles as C99, the library links from a C program and
+    validates its arguments there (no GPU needed: every check returns before
+    the first launch)."""
+    import shutil
+    import subprocess
+
+    if shutil.which("gcc") is None:
+        pytest.skip("no gcc")
+    from streamdiffusionv2_amd import _capi
+
+    here = os.path.dirname(os.path.abspath(__file__))
+    root = os.path.dirname(here)
+    exe = tmp_path / "abi_check"
+    lib_dir = str(_capi.LIB_PATH.parent)
+    build = subprocess.run(
+        ["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-I", os.path.join(root, "include"),
+         os.path.join(here, "c_abi", "abi_check.c"), "-o", str(exe), "-L", lib_dir, "-lsdv2kv",
+         "-L/opt/rocm/lib", "-Wl,-rpath," + lib_dir, "-Wl,-rpath,/opt/rocm/lib", "-Wl,--allow-shlib-undefined"],
+        capture_output=True, text=True)
+    assert build.returncode == 0, build.stderr
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert run.returncode == 0, run.stdout + run.stderr
+    assert "all checks passed" in run.stdout
+    assert "splits for 1x1560 tokens, 12 heads, 9360 keys: 3" in run.stdout
