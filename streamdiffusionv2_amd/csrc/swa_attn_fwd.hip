@@ -8,11 +8,15 @@
 // has to be unrolled.
 //
 // Work decomposition
-//   workgroup = 4 waves = 256 query rows of one (row, head), one workgroup per
-//   CU; wave w owns rows 64w..64w+63 as two 32-row blocks, so every K / V
-//   fragment fetched from LDS feeds two MFMAs.  Keys stream through LDS in
-//   tiles of 64 (K 16 KB + V 16 KB), three buffers each, filled two tiles
-//   ahead by global->LDS transfers that never touch registers.
+//   workgroup = 8 waves = 256 query rows of one (row, head), one workgroup per
+//   CU, two waves per SIMD with 256 registers each; wave w owns the 32-row
+//   block 32w..32w+31.  While one wave of a SIMD is held up (issuing its
+//   global->LDS transfers, at the barrier, waiting for an LDS fragment) the
+//   other keeps the matrix pipe fed; measured 3-6 % faster than four waves of
+//   two blocks each (512 registers, every LDS fragment feeding two MFMAs),
+//   which -DSDV2_FOUR_WAVES still builds.  Keys stream through LDS in tiles of
+//   64 (K 16 KB + V 16 KB), three buffers each, filled two tiles ahead by
+//   global->LDS transfers that never touch registers.
 //
 // Matrix layout (v_mfma_f32_32x32x16_bf16, D = A(32x16) * B(16x32) + C):
 //   S^T = K Q^T   A = K tile rows (ds_read_b128), B = Q, in registers for the
@@ -58,15 +62,25 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 typedef __attribute__((address_space(3))) char lds_char;
 
 constexpr int kD = SDV2_HEAD_DIM;           // 128
+#ifndef SDV2_FOUR_WAVES
+constexpr int kWaves = 8;                   // two waves per SIMD
+constexpr int kQB = 1;                      // 32-row query blocks per wave
+#define SDV2_Q_REG "a"                      // 256 registers per wave, at most 128 of them VGPRs: Q lives beside O
+#else
+#define SDV2_Q_REG "v"
 constexpr int kWaves = 4;
-constexpr int kThreads = kWaves * 64;
 constexpr int kQB = 2;                      // 32-row query blocks per wave
+#endif
+constexpr int kThreads = kWaves * 64;
+constexpr int kPieces = 16 / kWaves;        // global->LDS instructions per wave and matrix tile
 constexpr int kQRowsPerWave = 32 * kQB;
 constexpr int kQTile = kWaves * kQRowsPerWave;   // 256
 constexpr int kKTile = 64;
 constexpr int kTileBytes = kKTile * kD * 2;      // 16 KB per matrix
 constexpr int kStages = 3;
-constexpr int kLdsBytes = 2 * kStages * kTileBytes;   // 96 KB
+constexpr int kStageBytes = 16384;           // epilogue staging per wave: 32 rows x 512 B
+constexpr int kLdsBytes = 2 * kStages * kTileBytes > kWaves * kStageBytes ? 2 * kStages * kTileBytes
+                                                                         : kWaves * kStageBytes;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kCuSlots = 256;               // one workgroup per CU
 constexpr int kMaxDevices = 64;
@@ -161,7 +175,7 @@ __device__ __forceinline__ u32x2 lds_read_tr16_b64(uint32_t addr) {
 __device__ __forceinline__ void pin(float& x) { asm volatile("" : "+v"(x)); }
 __device__ __forceinline__ void pin(uint32_t& x) { asm volatile("" : "+v"(x)); }
 
-// The MFMAs of the fast pass are asm as well.  With one wave per SIMD the
+// The MFMAs of the fast pass are asm as well.  Left to itself the
 // compiler keeps every MFMA accumulator in the accumulation registers, but the
 // scores feed the vector ALU (which cannot read those) while the output tile
 // never does until the epilogue; naming the register class per product puts S
@@ -175,17 +189,17 @@ template <int kPending>
 __device__ __forceinline__ void mfma_s_first(f32x16& d, const u32x4& a, const bf16x8& b) {
   if constexpr (kPending >= 0)
     asm volatile("s_waitcnt lgkmcnt(%3)\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0"
-                 : "=&v"(d) : "v"(a), "v"(b), "n"(kPending));
+                 : "=&v"(d) : "v"(a), SDV2_Q_REG(b), "n"(kPending));
   else
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), SDV2_Q_REG(b));
 }
 template <int kPending>
 __device__ __forceinline__ void mfma_s(f32x16& d, const u32x4& a, const bf16x8& b) {
   if constexpr (kPending >= 0)
     asm volatile("s_waitcnt lgkmcnt(%3)\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0"
-                 : "+v"(d) : "v"(a), "v"(b), "n"(kPending));
+                 : "+v"(d) : "v"(a), SDV2_Q_REG(b), "n"(kPending));
   else
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), SDV2_Q_REG(b));
 }
 template <int kPending>
 __device__ __forceinline__ void mfma_o(f32x16& d, const u32x4& a, const u32x4& b) {
@@ -200,7 +214,7 @@ __device__ __forceinline__ void mfma_o(f32x16& d, const u32x4& a, const u32x4& b
 // Tile loader: global -> LDS without passing through registers
 // (global_load_lds_dwordx4).  One wave-wide instruction deposits 64 x 16 bytes
 // at consecutive LDS addresses, i.e. four 256-byte key rows.  Instruction i
-// (0..15, four per wave) fills rows 4i..4i+3; lane l lands on row 4i + l/16,
+// (0..15, kPieces per wave) fills rows 4i..4i+3; lane l lands on row 4i + l/16,
 // physical chunk l%16, so it must fetch logical chunk (l%16) ^ g(row).
 // ---------------------------------------------------------------------------
 // 16 bytes per lane from (wave-uniform base + this lane's 32-bit offset) to
@@ -220,20 +234,20 @@ __device__ __forceinline__ void dma16(const char* uniform_base, uint32_t lane_of
 // from the tile's first key row.  The last, partial tile redirects rows at or
 // past the valid length to the last valid key (their scores are masked), so
 // nothing outside the rows the caller declared valid is read.
-__device__ __forceinline__ void issue_matrix_tile(const char* base, uint32_t tok_bytes, const uint32_t (&off)[4],
+__device__ __forceinline__ void issue_matrix_tile(const char* base, uint32_t tok_bytes, const uint32_t (&off)[kPieces],
                                                   int key0, int seq, uint32_t lds_dst, int wave_u, int lane) {
   const char* tile = base + (int64_t)key0 * tok_bytes;      // wave-uniform
   if (key0 + kKTile <= seq) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) dma16(tile, off[j], lds_dst + (wave_u * 4 + j) * 1024);
+    for (int j = 0; j < kPieces; ++j) dma16(tile, off[j], lds_dst + (wave_u * kPieces + j) * 1024);
   } else {
     const int last_rel = seq - 1 - key0;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int r = 4 * (wave_u * 4 + j) + (lane >> 4);
+    for (int j = 0; j < kPieces; ++j) {
+      const int r = 4 * (wave_u * kPieces + j) + (lane >> 4);
       const int rr = r < last_rel ? r : last_rel;
       const uint32_t o = (uint32_t)rr * tok_bytes + (uint32_t)(((lane & 15) ^ swz(r)) << 4);
-      dma16(tile, o, lds_dst + (wave_u * 4 + j) * 1024);
+      dma16(tile, o, lds_dst + (wave_u * kPieces + j) * 1024);
     }
   }
 }
@@ -247,11 +261,17 @@ __device__ __forceinline__ void issue_matrix_tile(const char* base, uint32_t tok
 // behind the very moves they are meant to precede.
 template <int kTag>
 __device__ __forceinline__ void mfma_drain(f32x16 (&oacc)[kQB][4], f32x16 (&s)[2][kQB]) {
-  asm volatile("s_nop 15\n\ts_nop 15 ; matrix pipe drained, site %12"
-               : "+a"(oacc[0][0]), "+a"(oacc[0][1]), "+a"(oacc[0][2]), "+a"(oacc[0][3]), "+a"(oacc[1][0]),
-                 "+a"(oacc[1][1]), "+a"(oacc[1][2]), "+a"(oacc[1][3]), "+v"(s[0][0]), "+v"(s[0][1]),
-                 "+v"(s[1][0]), "+v"(s[1][1])
-               : "n"(kTag));
+  if constexpr (kQB == 2) {
+    asm volatile("s_nop 15\n\ts_nop 15 ; matrix pipe drained, site %12"
+                 : "+a"(oacc[0][0]), "+a"(oacc[0][1]), "+a"(oacc[0][2]), "+a"(oacc[0][3]), "+a"(oacc[kQB - 1][0]),
+                   "+a"(oacc[kQB - 1][1]), "+a"(oacc[kQB - 1][2]), "+a"(oacc[kQB - 1][3]), "+v"(s[0][0]),
+                   "+v"(s[0][kQB - 1]), "+v"(s[1][0]), "+v"(s[1][kQB - 1])
+                 : "n"(kTag));
+  } else {
+    asm volatile("s_nop 15\n\ts_nop 15 ; matrix pipe drained, site %6"
+                 : "+a"(oacc[0][0]), "+a"(oacc[0][1]), "+a"(oacc[0][2]), "+a"(oacc[0][3]), "+v"(s[0][0]), "+v"(s[1][0])
+                 : "n"(kTag));
+  }
 }
 
 struct LaneConst {
@@ -278,11 +298,11 @@ __device__ __forceinline__ void mask_block(f32x16& s, int key0, int seq, int hf,
 // ---------------------------------------------------------------------------
 // One pipeline slot of the fast pass.  Keys advance in blocks of 32; block j
 // goes through
-//   S(j)  = K_j Q^T            8 K fragments x 2 query blocks = 16 MFMAs
-//   SM(j) = exp2(scale * S)    VALU only, 2 x 16 scores per lane
-//   PV(j) = O^T += V_j^T P_j^T 8 V fragments x 2 query blocks = 16 MFMAs
+//   S(j)  = K_j Q^T            8 K fragments x kQB query blocks MFMAs
+//   SM(j) = exp2(scale * S)    VALU only, kQB x 16 scores per lane
+//   PV(j) = O^T += V_j^T P_j^T 8 V fragments x kQB query blocks MFMAs
 // and slot j runs S(j+1), SM(j) and PV(j-1) together: MFMAs of the two
-// products alternate (no accumulator is touched twice in a row) and the
+// products alternate (consecutive MFMAs never share an accumulator) and the
 // softmax instructions of block j are dealt out between them, so the matrix
 // pipe and the vector ALU of the wave work at the same time.  S(j) lives in
 // s[j&1], P(j) in p[j&1]; with the slot parity a template argument this is
@@ -340,28 +360,30 @@ __device__ __forceinline__ void slot(const LaneConst& c, const bf16x8 (&qf)[kQB]
   // A wave issues in order: a vector instruction only overlaps an MFMA if it
   // follows it in the stream, and it stalls the stream if it needs the result
   // of the instruction just before it.  So every MFMA is followed by a few
-  // softmax instructions that are independent of each other: the 32 scores of
-  // block j (both query blocks) flow through scale -> exp2 -> pack + row sum
-  // one step apart.  Score t belongs to group g = t/4: query block (t%4)/2,
+  // softmax instructions that are independent of each other: the 16 kQB scores
+  // of block j flow through scale -> exp2 -> pack + row sum one step apart.
+  // Score t belongs to group g = t / (2 kQB): query block (t % (2 kQB)) / 2,
   // accumulator register 2g + t%2.
-  float scaled[33], weight[33];
+  constexpr int kSPG = 2 * kQB;        // steps (= MFMAs) per fragment group: S of each block, PV of each block
+  constexpr int kSteps = 8 * kSPG;
+  float scaled[kSteps + 1], weight[kSteps + 1];
   auto score = [&](auto tc) -> float {
     constexpr int t = decltype(tc)::value;
-    return s_cur[(t & 3) >> 1][2 * (t >> 2) + (t & 1)];
+    return s_cur[(t % kSPG) >> 1][2 * (t / kSPG) + (t & 1)];
   };
   auto softmax_step = [&](auto tc) {
     constexpr int t = decltype(tc)::value;      // 0..33: stage 1 of score t, stage 2 of t-1, stage 3 of t-2
     if constexpr (kDoSM) {
-      if constexpr (t < 32) {
+      if constexpr (t < kSteps) {
         scaled[t] = score(tc) * c.c2;
         pin(scaled[t]);
       }
-      if constexpr (t >= 1 && t - 1 < 32) {
+      if constexpr (t >= 1 && t - 1 < kSteps) {
         weight[t - 1] = __builtin_amdgcn_exp2f(scaled[t - 1]);
         pin(weight[t - 1]);
       }
-      if constexpr (t >= 2 && t - 2 < 32 && ((t - 2) & 1) == 1) {
-        constexpr int u = t - 2, g = u >> 2, qb = (u & 3) >> 1;
+      if constexpr (t >= 2 && t - 2 < kSteps && ((t - 2) & 1) == 1) {
+        constexpr int u = t - 2, g = u / kSPG, qb = (u % kSPG) >> 1;
         uint32_t packed = pack_bf16x2(weight[u - 1], weight[u]);
         l[qb] = add_bf16_pair(packed, l[qb]);
         pin(packed);
@@ -371,29 +393,29 @@ __device__ __forceinline__ void slot(const LaneConst& c, const bf16x8 (&qf)[kQB]
     }
   };
 
-  static_for<32>([&](auto tc) {
+  static_for<kSteps>([&](auto tc) {
     constexpr int t = decltype(tc)::value;
-    constexpr int g = t >> 2, i = t & 3;
+    constexpr int g = t / kSPG, i = t % kSPG;
     constexpr int later = (g + kAhead < 8 ? kAhead : 7 - g) * kPerGroup;   // reads of later groups in flight
     constexpr int kk = g >> 2, db = g & 3;
     if constexpr (i == 0 && g + kAhead < 8) request(std::integral_constant<int, g + kAhead>{});
 
-    if constexpr (i == 0 && kDoS) {
-      if constexpr (g == 0) mfma_s_first<later + (kDoPV ? 2 : 0)>(s_nxt[0], kfrag[g], qf[0][g]);
-      else mfma_s<later + (kDoPV ? 2 : 0)>(s_nxt[0], kfrag[g], qf[0][g]);
+    if constexpr (i < kQB && kDoS) {
+      // the first MFMA on a fragment waits for it; the K fragment is followed by this group's two V reads
+      constexpr int pending = i == 0 ? later + (kDoPV ? 2 : 0) : -1;
+      if constexpr (g == 0) mfma_s_first<pending>(s_nxt[i], kfrag[g], qf[i][g]);
+      else mfma_s<pending>(s_nxt[i], kfrag[g], qf[i][g]);
     }
-    if constexpr (i == 1 && kDoS) {
-      if constexpr (g == 0) mfma_s_first<-1>(s_nxt[1], kfrag[g], qf[1][g]);
-      else mfma_s<-1>(s_nxt[1], kfrag[g], qf[1][g]);
+    if constexpr (i >= kQB && kDoPV) {
+      constexpr int qb = i - kQB;
+      mfma_o<(qb == 0 ? later : -1)>(oacc[qb][db], vfrag[g], p[kPar ^ 1][qb][kk]);
     }
-    if constexpr (i == 2 && kDoPV) mfma_o<later>(oacc[0][db], vfrag[g], p[kPar ^ 1][0][kk]);
-    if constexpr (i == 3 && kDoPV) mfma_o<-1>(oacc[1][db], vfrag[g], p[kPar ^ 1][1][kk]);
 
     softmax_step(tc);
     __builtin_amdgcn_sched_barrier(0);
   });
-  softmax_step(std::integral_constant<int, 32>{});
-  softmax_step(std::integral_constant<int, 33>{});
+  softmax_step(std::integral_constant<int, kSteps>{});
+  softmax_step(std::integral_constant<int, kSteps + 1>{});
 }
 
 // ---------------------------------------------------------------------------
@@ -404,7 +426,7 @@ __device__ __forceinline__ void slot(const LaneConst& c, const bf16x8 (&qf)[kQB]
 __device__ __forceinline__ void exact_pass(const AttnKernelArgs& a, const LaneConst& c, const bf16x8 (&qf)[kQB][8],
                                         f32x16 (&oacc)[kQB][4], float (&m_run)[kQB], float (&l_run)[kQB],
                                         const char* kbase, const char* vbase, uint32_t k_tok_bytes,
-                                        uint32_t v_tok_bytes, const uint32_t (&k_ld)[4], const uint32_t (&v_ld)[4],
+                                        uint32_t v_tok_bytes, const uint32_t (&k_ld)[kPieces], const uint32_t (&v_ld)[kPieces],
                                         int tile_begin, int n, int seq, uint32_t lds_addr0, lds_char* lds,
                                         int wave_u, int lane) {
 #pragma unroll
@@ -535,10 +557,10 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   const uint32_t k_tok_bytes = (uint32_t)(a.k_st.token * 2);
   const uint32_t v_tok_bytes = (uint32_t)(a.v_st.token * 2);
 
-  uint32_t k_ld[4], v_ld[4];
+  uint32_t k_ld[kPieces], v_ld[kPieces];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int r = 4 * (wave * 4 + j) + (lane >> 4);
+  for (int j = 0; j < kPieces; ++j) {
+    const int r = 4 * (wave * kPieces + j) + (lane >> 4);
     const int chunk = (lane & 15) ^ swz(r);
     k_ld[j] = (uint32_t)(r * k_tok_bytes + chunk * 16);
     v_ld[j] = (uint32_t)(r * v_tok_bytes + chunk * 16);
@@ -571,7 +593,11 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
     const int q_row_c = q_row[qb] < a.q_tokens ? q_row[qb] : a.q_tokens - 1;
     const uint16_t* qp = a.q + row * a.q_st.row + (int64_t)q_row_c * a.q_st.token + head * a.q_st.head + 8 * hf;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qf[qb][ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
+    for (int ks = 0; ks < 8; ++ks) {
+      qf[qb][ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
+      // the value is (re)defined in the register class every later use names, so it stays there
+      asm volatile("" : "+" SDV2_Q_REG(qf[qb][ks]));
+    }
   }
 
   // ---- per-lane LDS read addresses ------------------------------------------
@@ -630,8 +656,8 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
     for (int qb = 0; qb < kQB; ++qb)
 #pragma unroll
       for (int j = 0; j < 2; ++j) p[i][qb][j] = u32x4{0u, 0u, 0u, 0u};
-  float l_run[kQB] = {0.f, 0.f};     // this lane's share of each block's row sum
-  float m_run[kQB] = {0.f, 0.f};     // reference of the exponent: 0 in the fast pass
+  float l_run[kQB] = {};             // this lane's share of each block's row sum
+  float m_run[kQB] = {};             // reference of the exponent: 0 in the fast pass
   bool unsafe = false;
 
   // Tile T (64 keys) = blocks 2T, 2T+1, in K / V buffers T % 3.  Slot 2T needs
@@ -673,7 +699,7 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
     slot<kMask, 0, kLdsK(kB) + 32 * 256, kLdsVRel(kBPrev) + 32 * 256, true, true, true>(c, qf, s, p, oacc, l_run, key0,
                                                                                 key_end);
     if (T + 3 < n) {
-      __builtin_amdgcn_s_waitcnt(0x0F78);   // vmcnt(8)
+      __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kPieces));   // vmcnt: one K and one V tile's worth per wave
     } else {
       __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
     }
@@ -737,7 +763,7 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   // partial result of a split call (plus its log-sum-exp).  LDS operations of
   // one wave complete in order, so the block needs no barrier of its own.
   __syncthreads();                    // every wave is done with the K / V buffers
-  lds_char* stage = lds + wave * 16384;
+  lds_char* stage = lds + wave * kStageBytes;
   const int q0 = qtile * kQTile + wave * kQRowsPerWave;
 #pragma unroll
   for (int qb = 0; qb < kQB; ++qb) {
