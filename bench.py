@@ -53,6 +53,8 @@ def parse_args():
                     help="also time every chunk of a fresh stream while its ring fills (reported apart)")
     ap.add_argument("--qk-norm", action="store_true",
                     help="also time the append with the q/k RMSNorm folded in against torch norms + plain append")
+    ap.add_argument("--handoff", action="store_true",
+                    help="also time the owner change of a layer's cache block (export to / import from the wire layout)")
     ap.add_argument("--skip-mfma-reference", action="store_true",
                     help="do not time the vendor bf16 GEMM that shows what this box sustains on MFMA")
     return ap.parse_args()
@@ -277,6 +279,42 @@ def qk_norm_section(args, w):
     return out
 
 
+def handoff_section(args, w):
+    """Owner change of every layer's block: export (cache -> token-major wire)
+    and import (wire -> cache, indices shifted), one launch per tensor with the
+    library's timing events in each dispatch.  Bytes per launch = the tensor
+    read once and written once."""
+    from streamdiffusionv2_amd import handoff, ops, ring
+
+    dev = torch.device("cuda:0")
+    layers = min(w.layers, 4)
+    caches = ring.new_kv_cache(layers, 1, w.cache_tokens, w.heads, 1, dtype=w.dtype, device=dev)
+    if w.rows > 1:
+        ring.replicate_for_stream_batch(caches, w.rows)
+    for c in caches:
+        c["k"].normal_()
+        c["v"].normal_()
+    wires = [handoff.new_wire_like(c) for c in caches]
+    timer = ops.KernelTimer()
+    by = 2 * caches[0]["k"].numel() * caches[0]["k"].element_size()
+    out = {"bytes_per_launch": by, "layers_sampled": layers}
+    for name, pairs in (("export", [(wires[i].k, caches[i]["k"]) for i in range(layers)]),
+                        ("import", [(caches[i]["k"], wires[i].k) for i in range(layers)])):
+        for d, s_ in pairs:
+            ops.cache_relayout(d, s_)
+        ms = []
+        for _ in range(5):
+            for d, s_ in pairs:
+                ops.cache_relayout(d, s_, timer=timer)
+                ms.append(timer.elapsed_ms())
+        avg = sum(ms) / len(ms)
+        out[name + "_ms"] = avg
+        out[name + "_GBps"] = by / (avg * 1e-3) / 1e9
+    out["frac_of_hbm_peak"] = min(out["export_GBps"], out["import_GBps"]) / PEAK_HBM_GBS
+    timer.close()
+    return out
+
+
 def cpu_baseline(args, w):
     """The CPU oracle (a PyTorch restatement of the reference's op sequence)
     on this box's host cores: a bounded sample of steady-state chunks on a few
@@ -410,6 +448,8 @@ def main():
         result["fill_phase_ms_per_chunk"] = [round(x, 4) for x in g["fill_ms"]]
     if args.qk_norm:
         result["fused_qk_norm"] = qk_norm_section(args, w)
+    if args.handoff:
+        result["handoff"] = handoff_section(args, w)
     if not args.skip_mfma_reference:
         ref = mfma_reference()
         ref["attention_vs_random"] = achieved_tflops / ref["random"]

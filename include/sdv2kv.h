@@ -2,13 +2,14 @@
  * sdv2kv — C ABI of the MI355X (gfx950) ring-buffer KV-cache path for the
  * causal Wan DiT of StreamDiffusionV2.
  *
- * Three operators, all enqueued on a caller-supplied HIP stream, all working
+ * Four operators, all enqueued on a caller-supplied HIP stream, all working
  * on caller-owned device memory (the library owns nothing and keeps no
  * mutable state):
  *
  *   sdv2_kv_append_rope   fused RoPE-on-write chunk append
  *   sdv2_swa_attn_fwd     chunk-Q x (sink + window) K/V flash attention
  *   sdv2_sink_similarity  adaptive sink refresh decision
+ *   sdv2_cache_relayout   cache block <-> token-major wire format (owner change)
  *
  * Tensors are addressed as [rows, tokens, heads, 128] with explicit element
  * strides for the first three dimensions; the last dimension is contiguous.
@@ -30,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SDV2KV_ABI_VERSION 3
+#define SDV2KV_ABI_VERSION 4
 #define SDV2_HEAD_DIM 128      /* causal_stream_inference.py:99-100 fixes 128 */
 #define SDV2_MAX_ROWS 16       /* rows (B) per sdv2_kv_append_rope call       */
 #define SDV2_MAX_SINK_FRAMES 16 /* sink frames per sdv2_sink_similarity call  */
@@ -227,6 +228,44 @@ typedef struct sdv2_sink_sim_params {
 
 size_t sdv2_sink_similarity_workspace_bytes(int32_t rows, int32_t heads, int32_t sink_frames);
 int sdv2_sink_similarity(const sdv2_sink_sim_params* p);
+
+/* ------------------------------------------------------------------------
+ * Layout-changing copy of one layer's cache block, with the index hand-over.
+ *
+ * Serves the owner change of a block in the reference's pipeline-parallel
+ * mode, KVCacheManager.broadcast_kv_blocks
+ * (streamv2v/communication/kv_cache_manager.py:48-84): the donor's
+ * kv_cache1[i]["k"], ["v"], ["global_end_index"], ["local_end_index"] replace
+ * the receiver's (:70-78) and a receiver of lower rank then adds
+ * frame_seq_length * (donor - rank) * num_steps to global_end_index (:81-82).
+ * The transport itself (dist.broadcast) is the caller's; what travels is the
+ * reference's tensor, token-major contiguous [B, cap, H, 128].  This call
+ * produces that buffer from a cache in any stride order (src = cache, dst =
+ * wire) and absorbs it on the other side (src = wire, dst = cache):
+ *   dst[i, t, h, :] = src[i, t, h, :]
+ *   dst_global_end_index[i] = src_global_end_index[i] + global_end_shift
+ *   dst_local_end_index[i]  = src_local_end_index[i]
+ * The index part is skipped for a NULL dst pointer; tokens == 0 moves the
+ * indices only.  src and dst must not overlap.
+ * ---------------------------------------------------------------------- */
+typedef struct sdv2_relayout_params {
+  const void* src;             /* [B,cap,H,128]                                */
+  void* dst;
+  sdv2_stride3 src_stride, dst_stride;
+  int32_t dtype;               /* sdv2_dtype of both tensors                   */
+  int32_t rows, heads, head_dim;                  /* B, H, 128                 */
+  int64_t tokens;                                 /* cap                       */
+  const int64_t* src_global_end_index;            /* device int64 [B] or NULL  */
+  const int64_t* src_local_end_index;
+  int64_t* dst_global_end_index;                  /* device int64 [B] or NULL  */
+  int64_t* dst_local_end_index;
+  int64_t global_end_shift;
+  void* stream;                /* hipStream_t                                  */
+  void* timing_start;          /* optional timing events                       */
+  void* timing_stop;
+} sdv2_relayout_params;
+
+int sdv2_cache_relayout(const sdv2_relayout_params* p);
 
 /* ------------------------------------------------------------------------
  * Timing events.  No counterpart in the reference: they exist for

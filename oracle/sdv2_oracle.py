@@ -28,12 +28,17 @@ chunk_block_mask           models/wan/causal_model.py:670-686 (carried over to
                            cache positions)
 cross_attention_with_cache models/wan/wan_base/modules/model.py:160-196
 new_crossattn_cache        models/wan/causal_stream_inference.py:109-122
+compute_block_owners       streamv2v/communication/kv_cache_manager.py:86-108
+moved_blocks_by_donor      streamv2v/communication/kv_cache_manager.py:126-136
+receive_kv_block           streamv2v/communication/kv_cache_manager.py:66-82
 =========================  ====================================================
 
 Pinning (what fixes each function independently of this file) lives in
 ``tests/test_oracle_*.py`` (and, for the four functions at the end of the
 table, in ``tests/test_fused_qk_norm.py``, ``tests/test_block_mask.py``,
-``tests/test_cross_attention_cache.py``; the adaptive sink refresh inside
+``tests/test_cross_attention_cache.py``; the three block hand-off functions in
+``tests/test_handoff.py``, against the cases of the reference's own
+streamv2v/communication/test_communication.py:303-337 and hand-worked ones; the adaptive sink refresh inside
 ``RingAttentionOracle.step`` in ``tests/test_oracle_adaptive_sink.py``): closed forms for the tables, a scalar IEEE-double
 loop for the rotation and its double->float->bf16 rounding, hand traces of the
 slot schedule held as JSON under ``tests/golden/``, brute-force list
@@ -446,3 +451,45 @@ def noise_scale_and_step(
 def mix_noise(latents: torch.Tensor, noise: torch.Tensor, noise_scale: float) -> torch.Tensor:
     """noisy = noise*sigma + z*(1-sigma) (pipeline.py:310-314)."""
     return noise * noise_scale + latents * (1 - noise_scale)
+
+
+# --------------------------------------------------------------------------
+# Hand-off of a cache block between pipeline stages
+# --------------------------------------------------------------------------
+def compute_block_owners(block_intervals: torch.Tensor, total_blocks: int) -> torch.Tensor:
+    """Owner rank per block from [start, end) intervals per rank, -1 = nobody
+    (kv_cache_manager.py:98-106)."""
+    owners = torch.full((total_blocks,), -1, dtype=torch.int64)
+    for r in range(block_intervals.shape[0]):
+        s = int(block_intervals[r, 0].item())
+        e = int(block_intervals[r, 1].item())
+        if e > s:
+            owners[s:e] = r
+    return owners
+
+
+def moved_blocks_by_donor(old_block_intervals: torch.Tensor, new_block_intervals: torch.Tensor,
+                          total_blocks: int) -> dict:
+    """Blocks whose owner changes, keyed by the previous owner
+    (kv_cache_manager.py:126-136)."""
+    old = compute_block_owners(old_block_intervals, total_blocks)
+    new = compute_block_owners(new_block_intervals, total_blocks)
+    moved = {}
+    for i in range(total_blocks):
+        o, n = int(old[i].item()), int(new[i].item())
+        if o != n and o >= 0:
+            moved.setdefault(o, []).append(i)
+    return moved
+
+
+def receive_kv_block(entry: dict, donor_entry: dict, donor_rank: int, rank: int, frame_seq_length: int,
+                     time_step_length: int) -> None:
+    """What a rank's dict holds after ``broadcast_kv_blocks`` of one block
+    (kv_cache_manager.py:66-82): the donor's four tensors, copied in place, and
+    on a rank below the donor ``global_end_index`` moved on by
+    frame_seq_length * (donor - rank) * num_steps.  The donor itself
+    (rank == donor_rank) ends up unchanged."""
+    for name in ("k", "v", "global_end_index", "local_end_index"):
+        entry[name].copy_(donor_entry[name])
+    if donor_rank > rank:
+        entry["global_end_index"] += frame_seq_length * (donor_rank - rank) * time_step_length

@@ -11,7 +11,7 @@ from typing import Optional
 
 LIB_PATH = Path(__file__).resolve().parent / "_lib" / "libsdv2kv.so"
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 HEAD_DIM = 128
 MAX_ROWS = 16
 
@@ -37,6 +37,7 @@ EXPORTED_SYMBOLS = (
     "sdv2_swa_attn_fwd",
     "sdv2_sink_similarity_workspace_bytes",
     "sdv2_sink_similarity",
+    "sdv2_cache_relayout",
     "sdv2_event_create",
     "sdv2_event_destroy",
     "sdv2_event_elapsed_ms",
@@ -118,6 +119,21 @@ class SinkSimParams(C.Structure):
     ]
 
 
+class RelayoutParams(C.Structure):
+    _fields_ = [
+        ("src", C.c_void_p), ("dst", C.c_void_p),
+        ("src_stride", Stride3), ("dst_stride", Stride3),
+        ("dtype", C.c_int32),
+        ("rows", C.c_int32), ("heads", C.c_int32), ("head_dim", C.c_int32),
+        ("tokens", C.c_int64),
+        ("src_global_end_index", C.c_void_p), ("src_local_end_index", C.c_void_p),
+        ("dst_global_end_index", C.c_void_p), ("dst_local_end_index", C.c_void_p),
+        ("global_end_shift", C.c_int64),
+        ("stream", C.c_void_p),
+        ("timing_start", C.c_void_p), ("timing_stop", C.c_void_p),
+    ]
+
+
 _LIB: Optional[C.CDLL] = None
 
 
@@ -155,6 +171,8 @@ def lib() -> C.CDLL:
     handle.sdv2_sink_similarity_workspace_bytes.argtypes = [C.c_int32] * 3
     handle.sdv2_sink_similarity.restype = C.c_int
     handle.sdv2_sink_similarity.argtypes = [C.POINTER(SinkSimParams)]
+    handle.sdv2_cache_relayout.restype = C.c_int
+    handle.sdv2_cache_relayout.argtypes = [C.POINTER(RelayoutParams)]
     handle.sdv2_event_create.restype = C.c_int
     handle.sdv2_event_create.argtypes = [C.POINTER(C.c_void_p)]
     handle.sdv2_event_destroy.restype = C.c_int

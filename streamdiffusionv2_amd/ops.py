@@ -561,6 +561,47 @@ def flash_attention(q, k, v, q_lens=None, k_lens=None, dropout_p=0.0, softmax_sc
     return out if out_dtype == torch.bfloat16 else out.to(out_dtype)
 
 
+def cache_relayout(
+    dst: torch.Tensor,
+    src: torch.Tensor,
+    dst_indices: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+    src_indices: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
+    global_end_shift: int = 0,
+    timer: Optional["KernelTimer"] = None,
+) -> None:
+    """``dst[...] = src[...]`` for two [rows, cap, heads, 128] tensors in any
+    stride order, plus, with both index pairs (global_end_index,
+    local_end_index) given, ``dst_global = src_global + global_end_shift`` and
+    ``dst_local = src_local`` in the same launch: one side of the block
+    hand-off of streamv2v/communication/kv_cache_manager.py:66-82."""
+    flat = [dst, src] + list(dst_indices or ()) + list(src_indices or ())
+    dev = _require_gpu(*flat)
+    if src.dtype not in _DTYPES or dst.dtype != src.dtype:
+        raise RuntimeError(f"unsupported dtype pair {dst.dtype} / {src.dtype}")
+    if tuple(dst.shape) != tuple(src.shape):
+        raise RuntimeError(f"shape mismatch: {tuple(dst.shape)} vs {tuple(src.shape)}")
+    if (dst_indices is None) != (src_indices is None):
+        raise RuntimeError("index tensors are handed over as two pairs or not at all")
+    rows, tokens, heads, _ = src.shape
+    p = _capi.RelayoutParams()
+    p.src, p.src_stride = src.data_ptr(), _stride3(src, "src")
+    p.dst, p.dst_stride = dst.data_ptr(), _stride3(dst, "dst")
+    p.dtype = _DTYPES[src.dtype]
+    p.rows, p.heads, p.head_dim, p.tokens = rows, heads, HEAD_DIM, tokens
+    if dst_indices is not None:
+        for idx in (*dst_indices, *src_indices):
+            if idx.dtype != torch.int64 or idx.numel() < rows or not idx.is_contiguous():
+                raise RuntimeError("end-index tensors must be contiguous int64 with one entry per row")
+        p.dst_global_end_index, p.dst_local_end_index = (t.data_ptr() for t in dst_indices)
+        p.src_global_end_index, p.src_local_end_index = (t.data_ptr() for t in src_indices)
+        p.global_end_shift = int(global_end_shift)
+    p.stream = _stream_ptr(dev)
+    if timer is not None:
+        p.timing_start, p.timing_stop = timer.start, timer.stop
+    with torch.cuda.device(dev):
+        _capi.check(_capi.lib().sdv2_cache_relayout(C.byref(p)), "sdv2_cache_relayout")
+
+
 def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
     """Plain 16-byte-vector copy with the library's own kernel (used to scale
     hardware counters against a transfer of known size)."""

@@ -125,6 +125,13 @@ def _mirror(kv_cache: dict) -> _IndexMirror:
     return m
 
 
+def forget_index_mirror(kv_cache: dict) -> None:
+    """Drop the host copy of the two index tensors.  Needed after the library
+    itself rewrote them on the device (a raw kernel store does not bump the
+    tensors' version counters); the next plan reads them back once."""
+    kv_cache.pop(_MIRROR_KEY, None)
+
+
 @dataclass
 class AppendPlan:
     """What one layer call does, row by row."""

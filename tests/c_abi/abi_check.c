@@ -52,6 +52,19 @@ int main(void) {
   at.rows = 1; at.q_tokens = 8; at.max_seq_len = 8;
   expect("attention null tensors", sdv2_swa_attn_fwd(&at), SDV2_ERR_INVALID_ARG);
 
+  sdv2_relayout_params rl;
+  expect("relayout(NULL)", sdv2_cache_relayout(NULL), SDV2_ERR_INVALID_ARG);
+  memset(&rl, 0, sizeof rl);
+  rl.head_dim = 64;
+  expect("relayout head_dim 64", sdv2_cache_relayout(&rl), SDV2_ERR_UNSUPPORTED);
+  rl.head_dim = SDV2_HEAD_DIM;
+  expect("relayout of nothing", sdv2_cache_relayout(&rl), SDV2_OK);
+  rl.rows = 1; rl.tokens = 4; rl.heads = 2;
+  expect("relayout null tensors", sdv2_cache_relayout(&rl), SDV2_ERR_INVALID_ARG);
+  rl.tokens = 0;
+  rl.dst_global_end_index = (int64_t*)&rl;          /* destination index without a source */
+  expect("relayout index without source", sdv2_cache_relayout(&rl), SDV2_ERR_INVALID_ARG);
+
   printf("splits for 1x1560 tokens, 12 heads, 9360 keys: %d\n", sdv2_swa_attn_default_splits(1, 1560, 12, 9360));
   printf("workspace for that call: %zu bytes\n", sdv2_swa_attn_workspace_bytes(1, 1560, 12, 9360, 0));
   printf("sink-similarity workspace, 1 row, 12 heads, 3 sink frames: %zu bytes\n",
