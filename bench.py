@@ -53,6 +53,9 @@ def parse_args():
                     help="also time every chunk of a fresh stream while its ring fills (reported apart)")
     ap.add_argument("--qk-norm", action="store_true",
                     help="also time the append with the q/k RMSNorm folded in against torch norms + plain append")
+    ap.add_argument("--zero-inputs", action="store_true",
+                    help="all-zero q/k/v and caches: nothing toggles, the chip holds its top clock (a diagnostic of "
+                         "how much of the distance to the roofline is power, never a result)")
     ap.add_argument("--handoff", action="store_true",
                     help="also time the owner change of a layer's cache block (export to / import from the wire layout)")
     ap.add_argument("--skip-mfma-reference", action="store_true",
@@ -87,7 +90,7 @@ def gpu_bench(args, w):
     qkv = []
     for layer in range(w.layers):
         q, k, v = workloads.make_qkv(w, 0, layer)
-        qkv.append((q.to(dev), k.to(dev), v.to(dev)))
+        qkv.append(tuple(torch.zeros_like(t, device=dev) if args.zero_inputs else t.to(dev) for t in (q, k, v)))
     max_chunk = (1024 - w.grid[0]) // w.grid[0]     # keep the frame index inside the RoPE table
     state = {"call": 0}
 
@@ -138,7 +141,8 @@ def gpu_bench(args, w):
             cache["local_end_index"].data.copy_(torch.tensor(plan.new_local_end))
         for name in ("k", "v"):
             phys = cache[name].permute(0, 2, 1, 3)          # the head-major buffer itself
-            phys.copy_(torch.randn(phys.shape, generator=gen, device=dev, dtype=torch.float32) * w.input_scale)
+            if not args.zero_inputs:
+                phys.copy_(torch.randn(phys.shape, generator=gen, device=dev, dtype=torch.float32) * w.input_scale)
     state["call"] = fill_calls
     for _ in range(args.warmup):
         step()
@@ -413,7 +417,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
-        "data": "synthetic",
+        "data": "synthetic, all zeros (clock diagnostic, not a result)" if args.zero_inputs else "synthetic",
         "config": {
             "workload": w.name,
             "layers": w.layers, "rows": w.rows, "heads": w.heads, "head_dim": 128,
