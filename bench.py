@@ -56,6 +56,8 @@ def parse_args():
     ap.add_argument("--zero-inputs", action="store_true",
                     help="all-zero q/k/v and caches: nothing toggles, the chip holds its top clock (a diagnostic of "
                          "how much of the distance to the roofline is power, never a result)")
+    ap.add_argument("--adaptive-sink", action="store_true",
+                    help="also time the stream with the adaptive sink refresh on (one-frame chunks, one row)")
     ap.add_argument("--handoff", action="store_true",
                     help="also time the owner change of a layer's cache block (export to / import from the wire layout)")
     ap.add_argument("--skip-mfma-reference", action="store_true",
@@ -283,6 +285,46 @@ def qk_norm_section(args, w):
     return out
 
 
+def adaptive_sink_section(args, w):
+    """Steady-state chunks with the adaptive sink refresh on (sink 3, threshold
+    0.2: configs/wan_causal_dmd_v2v.yaml:55-56) against the same stream with it
+    off; applies to one-frame chunks only.  Wall-clock per chunk through the
+    public attend(), all layers."""
+    from streamdiffusionv2_amd import ring, workloads
+    from streamdiffusionv2_amd.attention import RingKVPath
+
+    if w.chunk_tokens != w.frame_tokens or w.rows != 1:
+        return {"skipped": "the refresh check only runs on one-frame chunks"}
+    dev = torch.device("cuda:0")
+    freqs = build_freqs()
+    S = w.chunk_tokens
+    grid = torch.tensor([list(w.grid)], dtype=torch.long)
+    qkv = [tuple(t.to(dev) for t in workloads.make_qkv(w, 0, layer)) for layer in range(w.layers)]
+    out = {"sink_size": 3}
+    fill = w.cache_tokens // S + 2
+    for name, thr in (("off_ms_per_step", -1.0), ("on_ms_per_step", 0.2)):
+        caches = ring.new_kv_cache(w.layers, 1, w.cache_tokens, w.heads, 1, dtype=w.dtype, device=dev)
+        paths = [RingKVPath(sink_size=3, adapt_sink_thr=thr) for _ in range(w.layers)]
+
+        def step(c):
+            for layer in range(w.layers):
+                q, k, v = qkv[layer]
+                paths[layer].attend(q, k, v, grid, freqs, caches[layer], [c * S])
+
+        for c in range(fill):
+            step(c)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for c in range(fill, fill + args.steps):
+            step(c)
+        torch.cuda.synchronize()
+        out[name] = (time.perf_counter() - t0) * 1e3 / args.steps
+        if thr > -1:
+            out["refreshes_in_last_step"] = sum(1 for p in paths if p.last_refresh and p.last_refresh[0] >= 0)
+    out["threshold"] = 0.2
+    return out
+
+
 def handoff_section(args, w):
     """Owner change of every layer's block: export (cache -> token-major wire)
     and import (wire -> cache, indices shifted), one launch per tensor with the
@@ -454,6 +496,8 @@ def main():
         result["fused_qk_norm"] = qk_norm_section(args, w)
     if args.handoff:
         result["handoff"] = handoff_section(args, w)
+    if args.adaptive_sink:
+        result["adaptive_sink"] = adaptive_sink_section(args, w)
     if not args.skip_mfma_reference:
         ref = mfma_reference()
         ref["attention_vs_random"] = achieved_tflops / ref["random"]

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SDV2KV_ABI_VERSION 4
+#define SDV2KV_ABI_VERSION 5
 #define SDV2_HEAD_DIM 128      /* causal_stream_inference.py:99-100 fixes 128 */
 #define SDV2_MAX_ROWS 16       /* rows (B) per sdv2_kv_append_rope call       */
 #define SDV2_MAX_SINK_FRAMES 16 /* sink frames per sdv2_sink_similarity call  */
@@ -122,6 +122,11 @@ typedef struct sdv2_append_params {
   float norm_eps;
   void* timing_start;          /* optional sdv2 timing events (see sdv2_event_create): */
   void* timing_stop;           /* recorded with the kernel's own dispatch              */
+  /* Optional slot chosen on the device: device int64 [B] or NULL.  A value
+   * >= 0 (and fitting the cache) replaces dst_start[i]; sdv2_sink_similarity
+   * writes it, so that an adaptive sink refresh needs no host round trip
+   * between the decision and the append.                                      */
+  const int64_t* dst_start_override;
 } sdv2_append_params;
 
 int sdv2_kv_append_rope(const sdv2_append_params* p);
@@ -224,6 +229,15 @@ typedef struct sdv2_sink_sim_params {
   void* workspace;             /* device scratch for the frame means           */
   size_t workspace_bytes;
   void* stream;                /* hipStream_t                                  */
+  /* Optional hand-over to the append that follows on the stream: device int64
+   * [B] or NULL.  Row i gets refresh[i] * tokens (the start of the refreshed
+   * sink frame: the slot (refresh + 1) * tokens at the head of the queue is
+   * where an evicting call writes, causal_model.py:297-306, 321-322) when it
+   * refreshes AND bit i of override_rows is set (= the caller's ring state
+   * says the row is on the evict branch; a row still filling writes at its
+   * fill position whatever the queue head is, :326-337), else -1.            */
+  int64_t* dst_start_override;
+  uint32_t override_rows;
 } sdv2_sink_sim_params;
 
 size_t sdv2_sink_similarity_workspace_bytes(int32_t rows, int32_t heads, int32_t sink_frames);

@@ -11,7 +11,7 @@ from typing import Optional
 
 LIB_PATH = Path(__file__).resolve().parent / "_lib" / "libsdv2kv.so"
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 HEAD_DIM = 128
 MAX_ROWS = 16
 
@@ -73,6 +73,7 @@ class AppendParams(C.Structure):
         ("norm_eps", C.c_float),
         ("timing_start", C.c_void_p),
         ("timing_stop", C.c_void_p),
+        ("dst_start_override", C.c_void_p),
     ]
 
 
@@ -116,6 +117,8 @@ class SinkSimParams(C.Structure):
         ("workspace", C.c_void_p),
         ("workspace_bytes", C.c_size_t),
         ("stream", C.c_void_p),
+        ("dst_start_override", C.c_void_p),
+        ("override_rows", C.c_uint32),
     ]
 
 

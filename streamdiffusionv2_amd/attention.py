@@ -69,7 +69,74 @@ class RingKVPath:
     def __init__(self, sink_size: int = 3, adapt_sink_thr: float = -1):
         self.sink_size = sink_size
         self.adapt_sink_thr = adapt_sink_thr
-        self.evict_idx: Optional[List[List[int]]] = None
+        self.evict_idx = None
+
+    # Ring state as the outside sees it.  With the adaptive sink refresh the
+    # decision of a call is made on the device and acted on there (the append
+    # that follows takes its slot from the decision kernel); the host picks it
+    # up when it next needs the state - normally a whole model pass later, when
+    # this layer is called again - so the stream never waits for a read-back.
+    # Reading any of the three attributes settles an outstanding decision first.
+    _evict_idx: Optional[List[List[int]]] = None
+    _last_plan = None
+    _last_refresh = None
+    _pending = None
+
+    @property
+    def evict_idx(self) -> Optional[List[List[int]]]:
+        self._settle()
+        return self._evict_idx
+
+    @evict_idx.setter
+    def evict_idx(self, value) -> None:
+        self._settle()
+        self._evict_idx = value
+
+    @property
+    def last_plan(self):
+        """The :class:`ring.AppendPlan` of the last call."""
+        self._settle()
+        return self._last_plan
+
+    @property
+    def last_refresh(self) -> Optional[List[int]]:
+        """Per row, the sink frame the last call's adaptive check chose to
+        overwrite (-1: none); None when the check did not run."""
+        self._settle()
+        return self._last_refresh
+
+    def settle(self) -> None:
+        """Make the host ring state current.  Call it before the cache dict of
+        this layer is re-sliced, replaced or handed to another owner."""
+        self._settle()
+
+    def _settle(self) -> None:
+        """Bring the host ring state up to date with the device's decision of
+        the last call.  A refresh puts (frame + 1) * frame_tokens at the head
+        of the row's queue before the call's own queue step
+        (causal_model.py:297-299, then :306-316 or :330-335); the end indices
+        and the pass counter do not depend on the queue, so the queue (and,
+        for an evicting row, the slot recorded in the plan) is all there is to
+        correct."""
+        pending = self._pending
+        if pending is None:
+            return
+        self._pending = None
+        pending["event"].synchronize()
+        refresh = pending["host"].tolist()
+        self._last_refresh = refresh
+        plan, tokens, frame_tokens = pending["plan"], pending["tokens"], pending["frame_tokens"]
+        sink_tokens = pending["sink_size"] * frame_tokens
+        for i, frame in enumerate(refresh):
+            if frame < 0:
+                continue
+            queue = list(pending["queues"][i])
+            queue.insert(0, (frame + 1) * frame_tokens)
+            dst_end = ring.advance_queue(queue, plan.evicting[i], plan.held[i], sink_tokens,
+                                         pending["starts"][i] + 2 * tokens, pending["cap"])
+            self._evict_idx[i][:] = queue
+            if plan.evicting[i]:
+                plan.dst_start[i] = dst_end - tokens      # where the decision kernel sent the append
 
     # 0 lets the library choose how many key ranges an attention call is split into
     num_splits = 0
@@ -78,6 +145,17 @@ class RingKVPath:
     # the cache and its chunk's blocks up to its own (the cache-less path's
     # kv_idx < ends[q_idx], causal_model.py:670-686).
     block_frames: Optional[int] = None
+
+    def _decision_buffers(self, rows: int, dev):
+        """Per path: the device slot override the decision kernel writes, the
+        pinned host copy of the decision and the event that says it arrived."""
+        buf = getattr(self, "_decision", None)
+        if buf is None or buf[0].numel() != rows or buf[0].device != dev:
+            buf = (torch.full((rows,), -1, dtype=torch.int64, device=dev),
+                   torch.empty((rows,), dtype=torch.int32, pin_memory=True),
+                   torch.cuda.Event())
+            self._decision = buf
+        return buf
 
     def _layer_launcher(self, q, k, v, kv_cache, table, grid, qk_norm=None):
         """The cached launch descriptors for this layer, rebuilt when the
@@ -110,17 +188,17 @@ class RingKVPath:
         if len(starts) != rows:
             raise RuntimeError(f"current_start has {len(starts)} entries for {rows} rows")
 
+        self._settle()
         cache_rows = kv_cache["k"].shape[0]
-        if self.evict_idx is None:
-            self.evict_idx = [[]]
-        if len(self.evict_idx) < cache_rows:
-            self.evict_idx = [list(self.evict_idx[0]) for _ in range(cache_rows)]
+        if self._evict_idx is None:
+            self._evict_idx = [[]]
+        if len(self._evict_idx) < cache_rows:
+            self._evict_idx = [list(self._evict_idx[0]) for _ in range(cache_rows)]
 
         table = ops.device_freqs(freqs, q.device)
-        self.last_refresh = None
-        if self.sink_size * frame_tokens > 0 and self.adapt_sink_thr > -1 and q.shape[1] <= frame_tokens:
-            # adaptive sink refresh (causal_model.py:284-299): one fused
-            # reduction on the device, one small read-back for all rows
+        self._last_refresh = None
+        adaptive = self.sink_size * frame_tokens > 0 and self.adapt_sink_thr > -1 and q.shape[1] <= frame_tokens
+        if adaptive:
             if qk_norm is not None:
                 raise RuntimeError("adaptive sink refresh reads the normalised key before the append: "
                                    "apply the q/k norm outside (qk_norm=None) in this mode")
@@ -128,22 +206,45 @@ class RingKVPath:
                 raise RuntimeError(
                     f"adaptive sink refresh needs one-frame chunks ({frame_tokens} tokens), got {q.shape[1]}"
                 )   # the reference's reshape(1, frame_seqlen, -1) fails the same way
-            _, refresh = ops.sink_similarity(
-                k, v, kv_cache["k"], kv_cache["v"], table, (h, w), [c // frame_tokens for c in starts],
-                self.sink_size, self.adapt_sink_thr)
-            self.last_refresh = refresh.tolist()
-            for i, frame in enumerate(self.last_refresh):
-                if frame >= 0:
-                    self.evict_idx[i].insert(0, (frame + 1) * frame_tokens)
+            evicting = ring.rows_evicting(kv_cache, starts, q.shape[1])
+            if any(e and not queue for e, queue in zip(evicting, self._evict_idx)):
+                # A full cache with an empty queue can only go on if this very call
+                # refreshes (otherwise causal_model.py:306 raises IndexError):
+                # the decision is needed before anything can be planned.
+                _, refresh = ops.sink_similarity(
+                    k, v, kv_cache["k"], kv_cache["v"], table, (h, w), [c // frame_tokens for c in starts],
+                    self.sink_size, self.adapt_sink_thr)
+                self._last_refresh = refresh.tolist()
+                for i, frame in enumerate(self._last_refresh):
+                    if frame >= 0:
+                        self._evict_idx[i].insert(0, (frame + 1) * frame_tokens)
+                adaptive = False
+            else:
+                queues_before = [list(queue) for queue in self._evict_idx]
 
-        plan = ring.plan_append(kv_cache, self.evict_idx, starts, q.shape[1], frame_tokens, self.sink_size)
+        # planned as if no row refreshed; _settle() corrects the host state later where one did
+        plan = ring.plan_append(kv_cache, self._evict_idx, starts, q.shape[1], frame_tokens, self.sink_size)
+        override = None
+        if adaptive:
+            # adaptive sink refresh (causal_model.py:284-299): one fused
+            # reduction on the device, whose decision goes straight to the
+            # append below and, written into pinned memory by the kernel, to the host
+            override, host, event = self._decision_buffers(rows, q.device)
+            ops.sink_similarity(
+                k, v, kv_cache["k"], kv_cache["v"], table, (h, w), [c // frame_tokens for c in starts],
+                self.sink_size, self.adapt_sink_thr, dst_start_override=override, override_rows=plan.evicting,
+                refresh_out=host)
+            event.record(torch.cuda.current_stream(q.device))
+            self._pending = dict(event=event, host=host, plan=plan, queues=queues_before, starts=list(starts),
+                                 tokens=q.shape[1], frame_tokens=frame_tokens, sink_size=self.sink_size,
+                                 cap=kv_cache["k"].shape[1])
         span = plan.max_seq_len
         seq = None
         if any(n != span for n in plan.new_local_end):
             # rows differ only while the stream batch is still filling; the
             # lengths are a handful of host ints, shipped asynchronously
             seq = torch.tensor(plan.new_local_end, dtype=torch.int32).to(q.device, non_blocking=True)
-        self.last_plan = plan
+        self._last_plan = plan
         mask_tokens = 0
         if self.block_frames is not None and self.block_frames * frame_tokens < q.shape[1]:
             mask_tokens = self.block_frames * frame_tokens
@@ -152,7 +253,7 @@ class RingKVPath:
             # steady-state fast path: launch descriptors are built once per
             # (cache, shape) and only patched per call
             launcher = self._layer_launcher(q, k, v, kv_cache, table, (f, h, w), qk_norm)
-            out = launcher.launch(q, k, v, [c // frame_tokens for c in starts], plan, seq, mask_tokens)
+            out = launcher.launch(q, k, v, [c // frame_tokens for c in starts], plan, seq, mask_tokens, override)
             if return_roped_query:
                 return out, launcher.roped_q.clone()
             return out
@@ -165,6 +266,7 @@ class RingKVPath:
             new_global_end=plan.new_global_end,
             new_local_end=plan.new_local_end,
             qk_norm=qk_norm,
+            dst_start_override=override,
         )
         mask = dict(chunk_key_start=list(plan.dst_start), mask_block_tokens=mask_tokens) if mask_tokens else {}
         if roped_q.dtype == torch.bfloat16:

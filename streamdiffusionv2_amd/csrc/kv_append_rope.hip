@@ -40,6 +40,8 @@ struct AppendKernelArgs {
   float norm_eps;
   int64_t* global_end;
   int64_t* local_end;
+  const int64_t* dst_override;              // device [rows] or null; a value >= 0 replaces dst_start[row]
+  int64_t cache_tokens;
   int32_t tokens, heads, grid_w, frame_tokens;
   int32_t split_t, split_h;                 // pair index bounds: [0,split_t) temporal, [split_t,split_h) height
   int32_t pairs;                            // 64
@@ -48,6 +50,18 @@ struct AppendKernelArgs {
   int64_t new_global[SDV2_MAX_ROWS];
   int64_t new_local[SDV2_MAX_ROWS];
 };
+
+// First cache token of the row's write: the host's choice unless a kernel
+// earlier on the stream (the adaptive sink decision) has put a slot into
+// dst_override.  A value that would not fit the cache is ignored.
+__device__ __forceinline__ int64_t row_dst_start(const AppendKernelArgs& a, int row) {
+  int64_t dst = a.dst_start[row];
+  if (a.dst_override) {
+    const int64_t o = a.dst_override[row];
+    if (o >= 0 && o + a.tokens <= a.cache_tokens) dst = o;
+  }
+  return dst;
+}
 
 template <typename T, bool kWithQ>
 __global__ __launch_bounds__(kLanesPerRow * kTokensPerBlock)
@@ -73,7 +87,7 @@ void kv_append_rope_kernel(const AppendKernelArgs a) {
   sdv2::load_rotation(a.freqs, a.pairs, a.split_t, a.split_h, lane, frame, hi, wi, cs);
 
   const int64_t e0 = lane * 8;
-  const int64_t dst_tok = a.dst_start[row] + tok;
+  const int64_t dst_tok = row_dst_start(a, row) + tok;
   const T* qi = static_cast<const T*>(a.q_in) + row * a.q_in_st.row + tok * a.q_in_st.token + e0;
   const T* ki = static_cast<const T*>(a.k_in) + row * a.k_in_st.row + tok * a.k_in_st.token + e0;
   const T* vi = static_cast<const T*>(a.v_in) + row * a.v_in_st.row + tok * a.v_in_st.token + e0;
@@ -150,7 +164,7 @@ void kv_append_norm_rope_kernel(const AppendKernelArgs a) {
   sdv2::load_rotation(a.freqs, a.pairs, a.split_t, a.split_h, sub, a.start_frame[row] + fi, hi, wi, cs);
 
   const int64_t e0 = sub * 8;
-  const int64_t dst_tok = a.dst_start[row] + tok;
+  const int64_t dst_tok = row_dst_start(a, row) + tok;
   const T* qi = static_cast<const T*>(a.q_in) + row * a.q_in_st.row + tok * a.q_in_st.token + e0;
   const T* ki = static_cast<const T*>(a.k_in) + row * a.k_in_st.row + tok * a.k_in_st.token + e0;
   const T* vi = static_cast<const T*>(a.v_in) + row * a.v_in_st.row + tok * a.v_in_st.token + e0;
@@ -256,6 +270,8 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
   a.q_norm_w = p->q_norm_weight; a.k_norm_w = p->k_norm_weight; a.norm_eps = p->norm_eps;
   a.global_end = p->global_end_index;
   a.local_end = p->local_end_index;
+  a.dst_override = p->dst_start_override;
+  a.cache_tokens = p->cache_tokens;
   a.tokens = p->tokens; a.heads = p->heads; a.grid_w = p->grid_w;
   a.frame_tokens = p->grid_h * p->grid_w;
   a.pairs = p->head_dim / 2;

@@ -6,10 +6,15 @@
 // incoming one-frame chunk's roped K and its V; the two similarities are
 // averaged and, when the smallest falls below the threshold, that sink frame
 // is to be overwritten next.  The reference does this with four reductions and
-// two host round trips per row; here one reduction kernel produces every frame
-// mean (rotating the new keys on the fly with the append kernel's arithmetic,
-// so they never have to be staged) and a second, tiny kernel turns the means
-// into similarities and the decision.  The caller reads back one int per row.
+// two host round trips per row; here one reduction kernel sums every frame
+// over its tokens, eight token ranges per (frame, head) side by side (rotating
+// the new keys on the fly with the append kernel's arithmetic, so they never
+// have to be staged), and a second, tiny kernel turns the sums into means,
+// similarities and the decision.  The caller reads back one int per row
+// - not necessarily at once: the decision kernel can also hand the slot a
+// refresh selects straight to the append kernel that follows it on the stream
+// (dst_start_override), so the host may pick the decision up a whole model
+// pass later, when it plans this layer's next call.
 //
 // Rounding follows the storage dtype: with bf16 tensors the frame means, the
 // two cosine similarities and their sum are each rounded to bf16 (they are
@@ -26,6 +31,9 @@ namespace {
 
 constexpr int kLanesPerRow = 16;            // 16 lanes x 8 elements = 128
 constexpr int kTokenLanes = 16;             // 256 threads
+constexpr int kTokenSplits = 8;             // workgroups per (frame, head): token ranges summed apart
+constexpr int kMaxHeads = 64;
+constexpr int kDecideThreads = 1024;
 
 struct SinkSimKernelArgs {
   const void* k_in;
@@ -34,9 +42,11 @@ struct SinkSimKernelArgs {
   const void* v_cache;
   sdv2_stride3 k_in_st, v_in_st, k_st, v_st;
   const double2* freqs;
-  float* means;                             // [rows][2*sink+2][heads*128]
+  float* sums;                              // [rows][2*sink+2][kTokenSplits][heads*128]: token sums
   float* similarity;                        // [rows][sink]
   int32_t* refresh;                         // [rows]
+  int64_t* dst_override;                    // [rows] or null: slot start for the append that follows
+  uint32_t override_rows;                   // bit i: row i is about to evict, so a refresh moves its write
   int32_t tokens, heads, grid_w, sink_frames;
   int32_t split_t, split_h, pairs;
   float threshold;
@@ -52,17 +62,20 @@ __device__ __forceinline__ float round_to_storage<uint16_t>(float x) {
 template <>
 __device__ __forceinline__ float round_to_storage<float>(float x) { return x; }
 
-// grid (heads, 2*sink+2, rows): one workgroup reduces one head's 128 columns
-// of one frame over its tokens.
+// grid (heads, 2*sink+2, rows * kTokenSplits): one workgroup sums one head's
+// 128 columns of one frame over one eighth of its tokens.  (One workgroup per
+// frame and head would leave most of the chip idle: 96 workgroups for three
+// sink frames of twelve heads.)
 template <typename T>
 __global__ __launch_bounds__(kLanesPerRow * kTokenLanes)
-void sink_frame_mean_kernel(const SinkSimKernelArgs a) {
+void sink_frame_sum_kernel(const SinkSimKernelArgs a) {
   __shared__ float part[kTokenLanes][kLanesPerRow * 8];
   const int lane = threadIdx.x & (kLanesPerRow - 1);
   const int tl = threadIdx.x >> 4;
   const int head = blockIdx.x;
   const int m = blockIdx.y;
-  const int row = blockIdx.z;
+  const int row = blockIdx.z / kTokenSplits;
+  const int split = blockIdx.z - row * kTokenSplits;
   const int sink = a.sink_frames;
 
   const bool is_new = m >= 2 * sink;
@@ -72,18 +85,56 @@ void sink_frame_mean_kernel(const SinkSimKernelArgs a) {
   const T* base = static_cast<const T*>(is_new ? (is_k ? a.k_in : a.v_in) : (is_k ? a.k_cache : a.v_cache));
   base += row * st.row + static_cast<int64_t>(frame) * a.tokens * st.token + head * st.head + lane * 8;
 
+  const int per = (a.tokens + kTokenSplits - 1) / kTokenSplits;
+  const int t_end = (split + 1) * per < a.tokens ? (split + 1) * per : a.tokens;
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  for (int t = tl; t < a.tokens; t += kTokenLanes) {
-    sdv2::Vec8<T> x = sdv2::Vec8<T>::load(base + t * st.token);
-    if (is_new && is_k) {
+  constexpr int kUnroll = 4;
+  if (is_new && is_k) {
+    // the new keys are rotated on the way in; four tokens per trip, loads (data and table) issued together
+    auto rotation = [&](int t, double2 (&cs)[4]) {
       const int hi = t / a.grid_w;
-      const int wi = t - hi * a.grid_w;
-      double2 cs[4];
-      sdv2::load_rotation(a.freqs, a.pairs, a.split_t, a.split_h, lane, a.start_frame[row], hi, wi, cs);
-      x = sdv2::rotate(x, cs);
-    }
+      sdv2::load_rotation(a.freqs, a.pairs, a.split_t, a.split_h, lane, a.start_frame[row], hi, t - hi * a.grid_w, cs);
+    };
+    int t = split * per + tl;
+    for (; t + (kUnroll - 1) * kTokenLanes < t_end; t += kUnroll * kTokenLanes) {
+      sdv2::Vec8<T> x[kUnroll];
+      double2 cs[kUnroll][4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] += static_cast<float>(x.get(i));
+      for (int u = 0; u < kUnroll; ++u) {
+        x[u] = sdv2::Vec8<T>::load(base + (t + u * kTokenLanes) * st.token);
+        rotation(t + u * kTokenLanes, cs[u]);
+      }
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) {
+        const sdv2::Vec8<T> y = sdv2::rotate(x[u], cs[u]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] += static_cast<float>(y.get(i));
+      }
+    }
+    for (; t < t_end; t += kTokenLanes) {
+      double2 cs[4];
+      rotation(t, cs);
+      const sdv2::Vec8<T> y = sdv2::rotate(sdv2::Vec8<T>::load(base + t * st.token), cs);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] += static_cast<float>(y.get(i));
+    }
+  } else {
+    // four tokens per trip, their loads issued together; the order of the adds is the token order
+    int t = split * per + tl;
+    for (; t + (kUnroll - 1) * kTokenLanes < t_end; t += kUnroll * kTokenLanes) {
+      sdv2::Vec8<T> x[kUnroll];
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u) x[u] = sdv2::Vec8<T>::load(base + (t + u * kTokenLanes) * st.token);
+#pragma unroll
+      for (int u = 0; u < kUnroll; ++u)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] += static_cast<float>(x[u].get(i));
+    }
+    for (; t < t_end; t += kTokenLanes) {
+      const sdv2::Vec8<T> x = sdv2::Vec8<T>::load(base + t * st.token);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] += static_cast<float>(x.get(i));
+    }
   }
 #pragma unroll
   for (int i = 0; i < 8; ++i) part[tl][lane * 8 + i] = acc[i];
@@ -92,69 +143,124 @@ void sink_frame_mean_kernel(const SinkSimKernelArgs a) {
     float s = 0.f;
 #pragma unroll
     for (int j = 0; j < kTokenLanes; ++j) s += part[j][threadIdx.x];
-    const float mean = round_to_storage<T>(s * (1.0f / static_cast<float>(a.tokens)));
     const int64_t width = static_cast<int64_t>(a.heads) * 128;
-    a.means[(static_cast<int64_t>(row) * (2 * sink + 2) + m) * width + head * 128 + threadIdx.x] = mean;
+    a.sums[((static_cast<int64_t>(row) * (2 * sink + 2) + m) * kTokenSplits + split) * width + head * 128 +
+           threadIdx.x] = s;
   }
 }
 
-// sum over the workgroup in a fixed order; result valid in every thread
-__device__ __forceinline__ float block_sum(float x, float* scratch) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) x += __shfl_xor(x, off, 64);
-  __syncthreads();
-  if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = x;
-  __syncthreads();
-  return (scratch[0] + scratch[1]) + (scratch[2] + scratch[3]);
-}
-
-// grid (rows): cosine similarities, their average, the decision.
-template <typename T>
-__global__ __launch_bounds__(256)
+// grid (rows): frame means from the partial sums, cosine similarities, their
+// average, the decision.  One workgroup of 1024 threads per row; a thread owns
+// kCols columns (columns past the width are clamped and weighted with zero
+// instead of branched around, so all loads of a frame are issued together).
+// Every dot product is reduced inside its wave as soon as it is formed and the
+// per-wave results wait in LDS, so nothing but loads and arithmetic sits
+// between two frames; the workgroup synchronises once, before the tail.
+template <typename T, int kCols>
+__global__ __launch_bounds__(kDecideThreads)
 void sink_decide_kernel(const SinkSimKernelArgs a) {
-  __shared__ float scratch[4];
+  constexpr int kWaves = kDecideThreads / 64;
+  __shared__ float wave_part[SDV2_MAX_SINK_FRAMES + 1][kWaves][4];
+  __shared__ float sims[SDV2_MAX_SINK_FRAMES];
   const int row = blockIdx.x;
   const int sink = a.sink_frames;
   const int width = a.heads * 128;
-  const float* means = a.means + static_cast<int64_t>(row) * (2 * sink + 2) * width;
-  const float* k_new = means + static_cast<int64_t>(2 * sink) * width;
-  const float* v_new = k_new + width;
+  const float* sums = a.sums + static_cast<int64_t>(row) * (2 * sink + 2) * kTokenSplits * width;
+  const float inv_tokens = 1.0f / static_cast<float>(a.tokens);
   constexpr float kEps = 1e-8f;             // torch.cosine_similarity default
-
-  float kk = 0.f, vv = 0.f;
-  for (int c = threadIdx.x; c < width; c += 256) {
-    kk += k_new[c] * k_new[c];
-    vv += v_new[c] * v_new[c];
+  int col[kCols];
+  float live[kCols];
+#pragma unroll
+  for (int i = 0; i < kCols; ++i) {
+    const int c = threadIdx.x + i * kDecideThreads;
+    col[i] = c < width ? c : width - 1;
+    live[i] = c < width ? 1.f : 0.f;
   }
-  const float k_new_norm = fmaxf(sqrtf(block_sum(kk, scratch)), kEps);
-  const float v_new_norm = fmaxf(sqrtf(block_sum(vv, scratch)), kEps);
+  // means of frame m at this thread's columns: the token ranges in order, then the rounding of a stored mean
+  auto means = [&](int m, float (&out)[kCols]) {
+    const float* p = sums + static_cast<int64_t>(m) * kTokenSplits * width;
+    float part[kCols][kTokenSplits];
+#pragma unroll
+    for (int i = 0; i < kCols; ++i)
+#pragma unroll
+      for (int j = 0; j < kTokenSplits; ++j) part[i][j] = p[static_cast<int64_t>(j) * width + col[i]];
+#pragma unroll
+    for (int i = 0; i < kCols; ++i) {
+      float s = 0.f;
+#pragma unroll
+      for (int j = 0; j < kTokenSplits; ++j) s += part[i][j];
+      out[i] = round_to_storage<T>(s * inv_tokens) * live[i];
+    }
+  };
+  // this wave's share of four sums, in a fixed order, parked in LDS
+  auto park = [&](int slot, float (&x)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) x[i] += __shfl_xor(x[i], off, 64);
+    if ((threadIdx.x & 63) == 0)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) wave_part[slot][threadIdx.x >> 6][i] = x[i];
+  };
+  auto total = [&](int slot, int i) {
+    float s = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) s += wave_part[slot][w][i];
+    return s;
+  };
 
-  float best = 0.f;
-  int best_frame = -1;
+  float k_new[kCols], v_new[kCols];
+  means(2 * sink, k_new);
+  means(2 * sink + 1, v_new);
+  float n[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < kCols; ++i) {
+    n[0] += k_new[i] * k_new[i];
+    n[1] += v_new[i] * v_new[i];
+  }
+  park(sink, n);
   for (int j = 0; j < sink; ++j) {
-    const float* ks = means + static_cast<int64_t>(j) * width;
-    const float* vs = means + static_cast<int64_t>(sink + j) * width;
-    float dk = 0.f, nk = 0.f, dv = 0.f, nv = 0.f;
-    for (int c = threadIdx.x; c < width; c += 256) {
-      dk += ks[c] * k_new[c];
-      nk += ks[c] * ks[c];
-      dv += vs[c] * v_new[c];
-      nv += vs[c] * vs[c];
+    float ks[kCols], vs[kCols];
+    means(j, ks);
+    means(sink + j, vs);
+    float d[4] = {0.f, 0.f, 0.f, 0.f};      // k.k_new, |k|^2, v.v_new, |v|^2
+#pragma unroll
+    for (int i = 0; i < kCols; ++i) {
+      d[0] += ks[i] * k_new[i];
+      d[1] += ks[i] * ks[i];
+      d[2] += vs[i] * v_new[i];
+      d[3] += vs[i] * vs[i];
     }
-    dk = block_sum(dk, scratch);
-    nk = block_sum(nk, scratch);
-    dv = block_sum(dv, scratch);
-    nv = block_sum(nv, scratch);
-    const float cos_k = round_to_storage<T>(dk / (fmaxf(sqrtf(nk), kEps) * k_new_norm));
-    const float cos_v = round_to_storage<T>(dv / (fmaxf(sqrtf(nv), kEps) * v_new_norm));
-    const float sim = round_to_storage<T>(cos_k + cos_v) * 0.5f;
-    if (threadIdx.x == 0) a.similarity[row * sink + j] = sim;
-    if (best_frame < 0 || sim < best) {       // first minimum, as torch.argmin
-      best = sim;
-      best_frame = j;
-    }
+    park(j, d);
   }
-  if (threadIdx.x == 0) a.refresh[row] = best < round_to_storage<T>(a.threshold) ? best_frame : -1;
+  __syncthreads();
+  if (threadIdx.x < sink) {
+    const int j = threadIdx.x;
+    const float k_new_norm = fmaxf(sqrtf(total(sink, 0)), kEps);
+    const float v_new_norm = fmaxf(sqrtf(total(sink, 1)), kEps);
+    const float cos_k = round_to_storage<T>(total(j, 0) / (fmaxf(sqrtf(total(j, 1)), kEps) * k_new_norm));
+    const float cos_v = round_to_storage<T>(total(j, 2) / (fmaxf(sqrtf(total(j, 3)), kEps) * v_new_norm));
+    const float sim = round_to_storage<T>(cos_k + cos_v) * 0.5f;
+    a.similarity[row * sink + j] = sim;
+    sims[j] = sim;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float best = sims[0];
+    int best_frame = 0;
+    for (int j = 1; j < sink; ++j)
+      if (sims[j] < best) {                   // first minimum, as torch.argmin
+        best = sims[j];
+        best_frame = j;
+      }
+    const int frame = best < round_to_storage<T>(a.threshold) ? best_frame : -1;
+    a.refresh[row] = frame;
+    // The refreshed sink frame goes to the head of the row's eviction queue
+    // (causal_model.py:297-299); a call on the evict branch then writes its
+    // one-frame chunk at [(frame + 1) * tokens - tokens, (frame + 1) * tokens).
+    if (a.dst_override)
+      a.dst_override[row] = frame >= 0 && ((a.override_rows >> row) & 1u) ? static_cast<int64_t>(frame) * a.tokens : -1;
+  }
 }
 
 bool stride_ok(const sdv2_stride3& s, int vec) {
@@ -167,7 +273,8 @@ bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 
 extern "C" size_t sdv2_sink_similarity_workspace_bytes(int32_t rows, int32_t heads, int32_t sink_frames) {
   if (rows <= 0 || heads <= 0 || sink_frames <= 0) return 0;
-  return static_cast<size_t>(rows) * (2 * static_cast<size_t>(sink_frames) + 2) * heads * SDV2_HEAD_DIM * sizeof(float);
+  return static_cast<size_t>(rows) * (2 * static_cast<size_t>(sink_frames) + 2) * kTokenSplits * heads * SDV2_HEAD_DIM *
+         sizeof(float);
 }
 
 extern "C" int sdv2_sink_similarity(const sdv2_sink_sim_params* p) {
@@ -175,6 +282,7 @@ extern "C" int sdv2_sink_similarity(const sdv2_sink_sim_params* p) {
   if (p->head_dim != SDV2_HEAD_DIM) return SDV2_ERR_UNSUPPORTED;
   if (p->dtype != SDV2_BF16 && p->dtype != SDV2_F32) return SDV2_ERR_UNSUPPORTED;
   if (p->rows <= 0 || p->rows > SDV2_MAX_ROWS || p->heads <= 0) return SDV2_ERR_INVALID_ARG;
+  if (p->heads > kMaxHeads) return SDV2_ERR_UNSUPPORTED;
   if (p->sink_frames <= 0 || p->sink_frames > SDV2_MAX_SINK_FRAMES) return SDV2_ERR_INVALID_ARG;
   if (p->grid_h <= 0 || p->grid_w <= 0) return SDV2_ERR_INVALID_ARG;
   // the reference's reshape(1, frame_seqlen, -1) only holds for a one-frame chunk
@@ -201,9 +309,11 @@ extern "C" int sdv2_sink_similarity(const sdv2_sink_sim_params* p) {
   a.k_in = p->k_in; a.v_in = p->v_in; a.k_cache = p->k_cache; a.v_cache = p->v_cache;
   a.k_in_st = p->k_in_stride; a.v_in_st = p->v_in_stride; a.k_st = p->k_cache_stride; a.v_st = p->v_cache_stride;
   a.freqs = reinterpret_cast<const double2*>(p->freqs);
-  a.means = static_cast<float*>(p->workspace);
+  a.sums = static_cast<float*>(p->workspace);
   a.similarity = p->similarity;
   a.refresh = p->refresh;
+  a.dst_override = p->dst_start_override;
+  a.override_rows = p->override_rows;
   a.tokens = p->tokens; a.heads = p->heads; a.grid_w = p->grid_w; a.sink_frames = p->sink_frames;
   a.pairs = p->head_dim / 2;
   const int third = a.pairs / 3;
@@ -214,14 +324,18 @@ extern "C" int sdv2_sink_similarity(const sdv2_sink_sim_params* p) {
 
   hipStream_t stream = static_cast<hipStream_t>(p->stream);
   const dim3 block(kLanesPerRow * kTokenLanes);
-  const dim3 grid_mean(p->heads, 2 * p->sink_frames + 2, p->rows);
+  const dim3 grid_mean(p->heads, 2 * p->sink_frames + 2, p->rows * kTokenSplits);
   const dim3 grid_decide(p->rows);
+  // columns per thread of the decision kernel: 2 up to 16 heads, 8 up to 64
+  const bool wide = p->heads * 128 > 2 * kDecideThreads;
   if (p->dtype == SDV2_BF16) {
-    hipLaunchKernelGGL(sink_frame_mean_kernel<uint16_t>, grid_mean, block, 0, stream, a);
-    hipLaunchKernelGGL(sink_decide_kernel<uint16_t>, grid_decide, dim3(256), 0, stream, a);
+    hipLaunchKernelGGL(sink_frame_sum_kernel<uint16_t>, grid_mean, block, 0, stream, a);
+    if (wide) hipLaunchKernelGGL((sink_decide_kernel<uint16_t, 8>), grid_decide, dim3(kDecideThreads), 0, stream, a);
+    else hipLaunchKernelGGL((sink_decide_kernel<uint16_t, 2>), grid_decide, dim3(kDecideThreads), 0, stream, a);
   } else {
-    hipLaunchKernelGGL(sink_frame_mean_kernel<float>, grid_mean, block, 0, stream, a);
-    hipLaunchKernelGGL(sink_decide_kernel<float>, grid_decide, dim3(256), 0, stream, a);
+    hipLaunchKernelGGL(sink_frame_sum_kernel<float>, grid_mean, block, 0, stream, a);
+    if (wide) hipLaunchKernelGGL((sink_decide_kernel<float, 8>), grid_decide, dim3(kDecideThreads), 0, stream, a);
+    else hipLaunchKernelGGL((sink_decide_kernel<float, 2>), grid_decide, dim3(kDecideThreads), 0, stream, a);
   }
   return hipGetLastError() == hipSuccess ? SDV2_OK : SDV2_ERR_LAUNCH;
 }

@@ -83,6 +83,11 @@ def _check_norm(qk_norm, dtype, heads: int, dev) -> None:
         raise RuntimeError("norm eps must be >= 0")
 
 
+def _check_override(t: torch.Tensor, rows: int, dev) -> None:
+    if t.dtype != torch.int64 or t.numel() < rows or not t.is_contiguous() or t.device != dev:
+        raise RuntimeError(f"dst_start_override must be a contiguous int64 tensor with one entry per row on {dev}")
+
+
 def kv_append_rope(
     q: Optional[torch.Tensor],
     k: torch.Tensor,
@@ -99,9 +104,14 @@ def kv_append_rope(
     new_global_end: Optional[Sequence[int]] = None,
     new_local_end: Optional[Sequence[int]] = None,
     qk_norm: Optional[Tuple[torch.Tensor, torch.Tensor, float]] = None,
+    dst_start_override: Optional[torch.Tensor] = None,
 ) -> Optional[torch.Tensor]:
     """RoPE q and k, write k' and v into the cache at ``dst_starts`` and store
     the new end indices.  Returns the roped query (``q_out`` or a new tensor).
+
+    ``dst_start_override`` (device int64 [B], written by
+    :func:`sink_similarity`) replaces ``dst_starts[i]`` where it holds a value
+    >= 0.
 
     ``qk_norm`` = (q weight, k weight, eps) folds the WanRMSNorm of the
     projection outputs in (wan_base/modules/model.py:70-86): q and k are then
@@ -135,6 +145,8 @@ def kv_append_rope(
         _check_norm(qk_norm, k.dtype, heads, dev)
         if q is None:
             raise RuntimeError("the fused q/k norm needs q")
+    if dst_start_override is not None:
+        _check_override(dst_start_override, rows, dev)
 
     lib = _capi.lib()
     stream = _stream_ptr(dev)
@@ -175,6 +187,8 @@ def kv_append_rope(
             if qk_norm is not None:
                 p.q_norm_weight, p.k_norm_weight = qk_norm[0].data_ptr(), qk_norm[1].data_ptr()
                 p.norm_eps = float(qk_norm[2])
+            if dst_start_override is not None:
+                p.dst_start_override = dst_start_override.data_ptr() + 8 * r0
             _capi.check(lib.sdv2_kv_append_rope(C.byref(p)), "sdv2_kv_append_rope")
     return q_out
 
@@ -287,9 +301,20 @@ def sink_similarity(
     start_frames: Sequence[int],
     sink_frames: int,
     threshold: float,
+    dst_start_override: Optional[torch.Tensor] = None,
+    override_rows: Sequence[bool] = (),
+    refresh_out: Optional[torch.Tensor] = None,
 ):
     """Adaptive sink refresh decision (causal_model.py:284-299) for a
     one-frame chunk, before its append.
+
+    With ``dst_start_override`` (device int64 [B]) the decision is also handed
+    to the append that follows on the stream: row i gets the start of the
+    refreshed sink frame when it refreshes and ``override_rows[i]`` says the
+    row is about to evict, else -1.  ``refresh_out`` (int32 [B]) receives the
+    decision instead of a new device tensor; it may be PINNED host memory, which
+    the kernel then writes directly (valid on the host once the stream has
+    passed this call).
 
     k is the chunk's key BEFORE RoPE, v its value, both [B,S,H,128]; the caches
     are read as they are.  Returns (similarity float32 [B, sink_frames],
@@ -311,7 +336,13 @@ def sink_similarity(
         ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
         _SIM_WORKSPACES[dev] = ws
     similarity = torch.empty((rows, sink_frames), dtype=torch.float32, device=dev)
-    refresh = torch.empty((rows,), dtype=torch.int32, device=dev)
+    if refresh_out is None:
+        refresh = torch.empty((rows,), dtype=torch.int32, device=dev)
+    else:
+        refresh = refresh_out
+        on_device = refresh.device == dev or (refresh.device.type == "cpu" and refresh.is_pinned())
+        if refresh.dtype != torch.int32 or refresh.numel() < rows or not refresh.is_contiguous() or not on_device:
+            raise RuntimeError(f"refresh_out must be a contiguous int32 tensor with one entry per row, on {dev} or pinned")
 
     p = _capi.SinkSimParams()
     p.k_in, p.k_in_stride = k.data_ptr(), _stride3(k, "k")
@@ -332,6 +363,12 @@ def sink_similarity(
     p.similarity, p.refresh = similarity.data_ptr(), refresh.data_ptr()
     p.workspace, p.workspace_bytes = ws.data_ptr(), ws.numel()
     p.stream = _stream_ptr(dev)
+    if dst_start_override is not None:
+        _check_override(dst_start_override, rows, dev)
+        if len(override_rows) != rows:
+            raise RuntimeError("override_rows needs one flag per row")
+        p.dst_start_override = dst_start_override.data_ptr()
+        p.override_rows = sum(1 << i for i, flag in enumerate(override_rows) if flag)
     with torch.cuda.device(dev):
         _capi.check(lib.sdv2_sink_similarity(C.byref(p)), "sdv2_sink_similarity")
     return similarity, refresh
@@ -457,10 +494,13 @@ class LayerLauncher:
                                   kv_cache["global_end_index"].data_ptr(), kv_cache["local_end_index"].data_ptr())
 
     def patch(self, q, k, v, start_frames, plan, seq_lens: Optional[torch.Tensor] = None,
-              mask_block_tokens: int = 0) -> torch.Tensor:
+              mask_block_tokens: int = 0, dst_start_override: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Fill in what changes from call to call and allocate the output
         [rows, S, H, 128]; nothing is launched."""
         ap, at = self.ap, self.at
+        if dst_start_override is not None:
+            _check_override(dst_start_override, self.rows, self.dev)
+        ap.dst_start_override = dst_start_override.data_ptr() if dst_start_override is not None else None
         at.mask_block_tokens = mask_block_tokens
         if mask_block_tokens:
             self.chunk_starts = chunk_starts_tensor(plan.dst_start, self.rows, self.tokens, plan.max_seq_len, self.dev)
@@ -510,10 +550,10 @@ class LayerLauncher:
         _capi.check(self.lib.sdv2_swa_attn_fwd(self.at_ref), "sdv2_swa_attn_fwd")
 
     def launch(self, q, k, v, start_frames, plan, seq_lens: Optional[torch.Tensor] = None,
-               mask_block_tokens: int = 0) -> torch.Tensor:
+               mask_block_tokens: int = 0, dst_start_override: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Append + attention for one call; returns the attention output
         [rows, S, H, 128].  The roped query stays in ``self.roped_q``."""
-        out = self.patch(q, k, v, start_frames, plan, seq_lens, mask_block_tokens)
+        out = self.patch(q, k, v, start_frames, plan, seq_lens, mask_block_tokens, dst_start_override)
         if _current_device_index() != self.dev.index:
             with torch.cuda.device(self.dev):
                 self.run_append()

@@ -125,6 +125,14 @@ def _mirror(kv_cache: dict) -> _IndexMirror:
     return m
 
 
+def rows_evicting(kv_cache: dict, current_start: Sequence[int], n_new: int) -> List[bool]:
+    """Which rows the next :func:`plan_append` sends down the evict branch
+    (causal_model.py:302)."""
+    cap = kv_cache["k"].shape[1]
+    m = _mirror(kv_cache)
+    return [int(c) + n_new > cap or m.local_end[i] >= cap for i, c in enumerate(current_start)]
+
+
 def forget_index_mirror(kv_cache: dict) -> None:
     """Drop the host copy of the two index tensors.  Needed after the library
     itself rewrote them on the device (a raw kernel store does not bump the
@@ -138,10 +146,31 @@ class AppendPlan:
     dst_start: List[int]      # first cache token written
     new_global_end: List[int]
     new_local_end: List[int]  # == seq_lens of the attention that follows
+    evicting: List[bool] = None   # row took the evict branch (wrote at the head of its queue)
+    held: List[bool] = None       # ... without rotating the queue (a pass before the last, causal_model.py:310-311)
 
     @property
     def max_seq_len(self) -> int:
         return max(self.new_local_end)
+
+
+def advance_queue(queue: List[int], evicting: bool, held: bool, sink_tokens: int, next_end: int, cap: int):
+    """What one call does to a row's eviction queue (causal_model.py:306-316,
+    330-335).  An evicting call writes the slot ending at the head of the queue
+    (returned; IndexError when there is none) and, unless the pass counter
+    holds it there, rotates the head to the tail - or drops it when it lies in
+    the sink, as a refreshed sink frame does.  A filling call queues the slot
+    after its own once that slot lies beyond the sink."""
+    if evicting:
+        dst_end = queue[0]
+        if not held:
+            head = queue.pop(0)
+            if head > sink_tokens:
+                queue.append(head)
+        return dst_end
+    if sink_tokens < next_end <= cap and (not queue or queue[-1] != next_end):
+        queue.append(next_end)
+    return None
 
 
 def plan_append(
@@ -170,27 +199,24 @@ def plan_append(
             f"current_start has {len(current_start)} rows but the cache indices have {len(m.local_end)}"
         )
 
-    dst_start, new_g, new_l = [], [], []
+    dst_start, new_g, new_l, evicting, held = [], [], [], [], []
     for i, c_start in enumerate(current_start):
         c_start = int(c_start)
         c_end = c_start + n_new
         queue = evict_idx[i]
-        if c_end > cap or m.local_end[i] >= cap:
+        evicting.append(c_end > cap or m.local_end[i] >= cap)
+        held.append(evicting[-1] and cache_rows == 1 and kv_cache["current_step"] > 1)
+        if evicting[-1]:
             m.global_end[i], m.local_end[i] = c_start, cap
-            dst_end = queue[0]
-            if cache_rows == 1 and kv_cache["current_step"] > 1:
+            dst_end = advance_queue(queue, True, held[-1], sink_tokens, 0, cap)
+            if held[-1]:
                 kv_cache["current_step"] -= 1
             else:
-                head = queue.pop(0)
-                if head > sink_tokens:
-                    queue.append(head)
                 kv_cache["current_step"] = kv_cache["total_steps"]
             local_new = cap
         else:
             local_new = m.local_end[i] + c_end - m.global_end[i]
-            next_end = c_end + n_new
-            if sink_tokens < next_end <= cap and (not queue or queue[-1] != next_end):
-                queue.append(next_end)
+            advance_queue(queue, False, False, sink_tokens, c_end + n_new, cap)
             dst_end = local_new
         start = dst_end - n_new
         if start < 0 or dst_end > cap:
@@ -199,7 +225,7 @@ def plan_append(
         new_g.append(c_end)
         new_l.append(local_new)
         m.global_end[i], m.local_end[i] = c_end, local_new
-    return AppendPlan(dst_start, new_g, new_l)
+    return AppendPlan(dst_start, new_g, new_l, evicting, held)
 
 
 def closed_form_slot(chunk: int, n_slots: int, n_permanent: int) -> int:

@@ -176,6 +176,12 @@ class KVStreamPipeline:
         return out
 
 
+    def _settle_paths(self) -> None:
+        for path in self.generator.paths:
+            settle = getattr(path, "settle", None)
+            if settle is not None:
+                settle()
+
     # -- demo/vid2vid.py:113-135 -------------------------------------------
     _CACHE_TENSORS = ("k", "v", "global_end_index", "local_end_index")
 
@@ -185,6 +191,7 @@ class KVStreamPipeline:
         are kept aside untouched.  Nothing is copied."""
         if self.active_mode == "wo_batch":
             return
+        self._settle_paths()               # host ring state current before the dicts are re-sliced
         self._batch_state_refs = {
             "kv_cache1": [{name: entry[name] for name in self._CACHE_TENSORS} for entry in self.kv_cache1],
             "hidden_states": self.hidden_states,
@@ -206,6 +213,7 @@ class KVStreamPipeline:
             return
         if self._batch_state_refs is None:
             raise RuntimeError("Cannot restore batch mode before batch state has been captured")
+        self._settle_paths()
         for entry, saved in zip(self.kv_cache1, self._batch_state_refs["kv_cache1"]):
             for name in self._CACHE_TENSORS:
                 t = saved[name]
