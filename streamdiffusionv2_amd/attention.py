@@ -157,6 +157,11 @@ class RingKVPath:
             self._decision = buf
         return buf
 
+    @staticmethod
+    def _mark_decision(event, dev) -> None:
+        """The decision is on the host once the stream has passed this point."""
+        event.record(torch.cuda.current_stream(dev))
+
     def _layer_launcher(self, q, k, v, kv_cache, table, grid, qk_norm=None):
         """The cached launch descriptors for this layer, rebuilt when the
         cache, the shapes, the grid or the norm weights change."""
@@ -234,7 +239,7 @@ class RingKVPath:
                 k, v, kv_cache["k"], kv_cache["v"], table, (h, w), [c // frame_tokens for c in starts],
                 self.sink_size, self.adapt_sink_thr, dst_start_override=override, override_rows=plan.evicting,
                 refresh_out=host)
-            event.record(torch.cuda.current_stream(q.device))
+            self._mark_decision(event, q.device)
             self._pending = dict(event=event, host=host, plan=plan, queues=queues_before, starts=list(starts),
                                  tokens=q.shape[1], frame_tokens=frame_tokens, sink_size=self.sink_size,
                                  cap=kv_cache["k"].shape[1])

@@ -19,7 +19,9 @@ several GPUs would broadcast the four wire tensors from the donor and here
 defaults to handing the donor's wire straight back.
 
 The eviction queues (``evict_idx``) are module state in the reference and are
-not part of its broadcast; they are not moved here either.
+not part of its broadcast; they are not moved here either.  With the adaptive
+sink refresh on, read a layer's ``evict_idx`` (or call its ``settle()``) before
+its block changes owner, so that no decision is still on its way to the host.
 """
 from __future__ import annotations
 
