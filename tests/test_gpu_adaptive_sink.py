@@ -141,6 +141,47 @@ def test_similarity_operator(gpu_device, dtype, tol, head_major):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("heads,sink", [(40, 3), (17, 16), (64, 2), (1, 1)])
+def test_similarity_operator_wide_and_deep(gpu_device, heads, sink):
+    """The decision kernel has a build for up to 16 heads and one for up to 64,
+    and room for 16 sink frames; the slot hand-over is checked on the way
+    (rows 0 and 2 flagged as evicting)."""
+    from streamdiffusionv2_amd import ops, rope
+
+    print(f"sink similarity operator: heads={heads} sink={sink}", flush=True)
+    rows, cap = 3, (sink + 2) * FT
+    gen = torch.Generator().manual_seed(heads * 100 + sink)
+    basis = torch.randn(3, heads * 128, generator=gen)
+    _, k, v = directed_chunk(gen, rows, heads, torch.bfloat16, basis)
+    ck = torch.cat([directed_chunk(gen, rows, heads, torch.bfloat16, basis)[1] for _ in range(sink + 2)], dim=1)
+    cv = torch.cat([directed_chunk(gen, rows, heads, torch.bfloat16, basis)[2] for _ in range(sink + 2)], dim=1)
+    start_frames = [5, 0, 11]
+    roped = oracle.causal_rope_apply(k, [GRID] * rows, oracle.build_freqs(), start_frames).type_as(v)
+    want = []
+    for r in range(rows):
+        def means(t, frames):
+            return t.reshape(frames, FT, -1).mean(1)
+        sk = torch.cosine_similarity(means(ck[r:r + 1, :sink * FT], sink), means(roped[r:r + 1], 1), dim=-1)
+        sv = torch.cosine_similarity(means(cv[r:r + 1, :sink * FT], sink), means(v[r:r + 1], 1), dim=-1)
+        want.append(((sk + sv) / 2).float())
+    want = torch.stack(want)
+    table = ops.device_freqs(rope.build_freqs(), gpu_device)
+    override = torch.full((rows,), 12345, dtype=torch.int64, device=gpu_device)
+    sim, refresh = ops.sink_similarity(k.to(gpu_device), v.to(gpu_device), ck.to(gpu_device), cv.to(gpu_device), table,
+                                       GRID[1:], start_frames, sink, 1.5, dst_start_override=override,
+                                       override_rows=[True, False, True])
+    torch.cuda.synchronize()
+    assert (sim.cpu() - want).abs().max().item() <= 1e-2, (sim.cpu(), want)
+    got = refresh.cpu().tolist()
+    assert got == sim.argmin(dim=1).cpu().tolist()            # threshold 1.5: always the minimum
+    assert override.cpu().tolist() == [got[0] * FT, -1, got[2] * FT]
+    for r in range(rows):
+        s = want[r].sort().values
+        if sink == 1 or (s[1] - s[0]).item() > MARGIN:
+            assert got[r] == int(want[r].argmin())
+
+
+@pytest.mark.gpu
 def test_similarity_operator_rejects_bad_calls(gpu_device):
     from streamdiffusionv2_amd import ops, rope
 
@@ -156,6 +197,15 @@ def test_similarity_operator_rejects_bad_calls(gpu_device):
         ops.sink_similarity(x, x, cache, cache, table, GRID[1:], [1024], 2, THR)
     with pytest.raises(RuntimeError):       # CPU tensors: no fallback
         ops.sink_similarity(x.cpu(), x.cpu(), cache.cpu(), cache.cpu(), table, GRID[1:], [0], 2, THR)
+    with pytest.raises(RuntimeError):       # slot hand-over without the per-row flags
+        ops.sink_similarity(x, x, cache, cache, table, GRID[1:], [0], 2, THR,
+                            dst_start_override=torch.zeros(1, dtype=torch.int64, device=gpu_device))
+    with pytest.raises(RuntimeError):       # decision into unpinned host memory
+        ops.sink_similarity(x, x, cache, cache, table, GRID[1:], [0], 2, THR, refresh_out=torch.zeros(1, dtype=torch.int32))
+    wide = torch.zeros(1, FT, 65, 128, dtype=torch.bfloat16, device=gpu_device)
+    wide_cache = torch.zeros(1, 4 * FT, 65, 128, dtype=torch.bfloat16, device=gpu_device)
+    with pytest.raises(RuntimeError):       # more heads than the decision kernel is built for
+        ops.sink_similarity(wide, wide, wide_cache, wide_cache, table, GRID[1:], [0], 2, THR)
 
 
 @pytest.mark.gpu
