@@ -666,7 +666,8 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   // K tile T and V tile T-1 are free: that is where the one barrier per tile
   // sits, followed by the requests for K tile T+3 and V tile T+2.  What the
   // next two slots read was requested two barriers earlier, so the wait before
-  // the barrier leaves the newest eight transfers in flight.
+  // the barrier leaves the newest 2 * kPieces transfers of the wave (one K and
+  // one V tile's worth) in flight.
   //
   // Every tile runs the same code and the loop body is three whole tiles with
   // a single way in and out, so the accumulators keep their registers from trip
@@ -950,7 +951,8 @@ extern "C" int sdv2_swa_attn_fwd(const sdv2_attn_params* p) {
   if (items > (1 << 28)) return SDV2_ERR_INVALID_ARG;
   dim3 grid((unsigned)(8 * ((items + 7) / 8)));
   if (p->stages != SDV2_STAGE_MERGE) {
-    // 96 KB of LDS is more than the static limit: ask for it once per device.
+    // The tile buffers (96 KB) or the epilogue staging (16 KB per wave) exceed the static limit:
+    // ask for the dynamic size once per device.
     // The kernel exists twice: the mask inside the chunk costs the plain
     // variant about 2 % even when it is off, so it gets its own code.
     static std::atomic<bool> lds_ready[kMaxDevices];
