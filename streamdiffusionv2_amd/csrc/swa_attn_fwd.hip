@@ -713,9 +713,27 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   using B1 = std::integral_constant<int, 1>;
   using B2 = std::integral_constant<int, 2>;
 
+  const bool idle = __builtin_amdgcn_readfirstlane(qtile * kQTile + wave * kQRowsPerWave >= a.q_tokens);
   if (n > 0) {
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();        // the first tiles and the Q fragments have arrived
+    if (idle) {
+      // No query row of this wave exists (the last query tile of a call is
+      // rarely full).  The wave still moves its share of every K / V tile and
+      // meets the others at every barrier, but issues no LDS read, MFMA or
+      // softmax instruction: on a chip that runs this kernel against its power
+      // limit, work on rows nobody reads would only lower the clock for the rest.
+      for (int T = 0; T < n; ++T) {
+        if (T + 3 < n) {
+          __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kPieces));
+        } else {
+          __builtin_amdgcn_s_waitcnt(0x0F70);
+        }
+        __syncthreads();
+        if (T + 3 < n) issue_k(T + 3, T % kStages);
+        if (T + 2 < n) issue_v(T + 2, (T + 2) % kStages);
+      }
+    } else {
     // S(0) alone fills the pipeline
     slot<kMask, 1, kLdsK(0), 0, true, false, false>(c, qf, s, p, oacc, l_run, 0, key_end);
     // Three tiles per trip, one per buffer; the last trip stops after the last
@@ -742,6 +760,7 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
     }
     mfma_drain<0>(oacc, s);
     unsafe = row_sums_unsafe();
+    }
 
     // Did any wave of the workgroup see an unsafe row sum?  (LDS is free now.)
     __syncthreads();
@@ -766,6 +785,7 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   __syncthreads();                    // every wave is done with the K / V buffers
   lds_char* stage = lds + wave * kStageBytes;
   const int q0 = qtile * kQTile + wave * kQRowsPerWave;
+  if (idle) return;
 #pragma unroll
   for (int qb = 0; qb < kQB; ++qb) {
     const float l_tot = half_sum(l_run[qb]);
