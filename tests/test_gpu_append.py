@@ -152,3 +152,54 @@ def test_append_random_shapes(gpu_device):
             assert g_idx.tolist() == list(range(5, 5 + rows)) and l_idx.tolist() == list(range(9, 9 + rows))
         else:
             assert g_idx.tolist() == [-1] * rows
+
+
+@pytest.mark.parametrize("fused_norm", [False, True])
+def test_append_slot_chosen_on_the_device(gpu_device, fused_norm):
+    """dst_start_override: a value >= 0 that fits the cache replaces the host's
+    slot for that row, -1 and values that would leave the cache do not (both
+    append kernels)."""
+    from streamdiffusionv2_amd import ops
+
+    print(f"append with a device-chosen slot, fused norm {fused_norm}", flush=True)
+    torch.manual_seed(7)
+    rows, grid, heads = 4, (1, 4, 6), 3
+    S = 24
+    cap = 5 * S
+    q, k, v = (torch.randn(rows, S, heads, 128).bfloat16() for _ in range(3))
+    start_frames = [2, 3, 4, 5]
+    host_dst = [S, 2 * S, 3 * S, 4 * S]
+    override = torch.tensor([0, -1, cap - S + 1, 2 * S], dtype=torch.int64)   # row 2 would overrun the cache
+    lands = [0, 2 * S, 3 * S, 2 * S]
+    weights = None
+    kn, qn = k, q
+    if fused_norm:
+        wq, wk = (torch.rand(heads * 128) + 0.5).bfloat16(), (torch.rand(heads * 128) + 0.5).bfloat16()
+        weights = (wq.to(gpu_device), wk.to(gpu_device), 1e-6)
+        qn = oracle.wan_rms_norm(q.flatten(2), wq, 1e-6).view_as(q)
+        kn = oracle.wan_rms_norm(k.flatten(2), wk, 1e-6).view_as(k)
+    want_k = oracle.causal_rope_apply(kn, [grid] * rows, oracle.build_freqs(), start_frames).type_as(v)
+    kc = torch.zeros(rows, heads, cap, 128, dtype=torch.bfloat16, device=gpu_device).permute(0, 2, 1, 3)
+    vc = torch.zeros(rows, heads, cap, 128, dtype=torch.bfloat16, device=gpu_device).permute(0, 2, 1, 3)
+    from streamdiffusionv2_amd import rope
+    table = ops.device_freqs(rope.build_freqs(), gpu_device)
+    ops.kv_append_rope(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), kc, vc, table, grid, start_frames, host_dst,
+                       qk_norm=weights, dst_start_override=override.to(gpu_device))
+    torch.cuda.synchronize()
+    for r in range(rows):
+        got_v = vc[r].cpu()
+        assert torch.equal(got_v[lands[r]:lands[r] + S], v[r]), r
+        untouched = torch.ones(cap, dtype=torch.bool)
+        untouched[lands[r]:lands[r] + S] = False
+        assert not got_v[untouched].any() and not kc[r].cpu()[untouched].any(), r
+        got_k = kc[r, lands[r]:lands[r] + S].cpu()
+        if fused_norm:      # the fused sum of squares may differ from torch's in the last place
+            assert (got_k.float() - want_k[r].float()).abs().max().item() <= 2 ** -6 * want_k[r].float().abs().max().item()
+        else:
+            assert torch.equal(_bits(got_k), _bits(want_k[r])), r
+    with pytest.raises(RuntimeError):       # wrong dtype
+        ops.kv_append_rope(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), kc, vc, table, grid, start_frames,
+                           host_dst, dst_start_override=override.int().to(gpu_device))
+    with pytest.raises(RuntimeError):       # not on the device
+        ops.kv_append_rope(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), kc, vc, table, grid, start_frames,
+                           host_dst, dst_start_override=override)
