@@ -602,8 +602,9 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       qf[qb][ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
-      // the value is (re)defined in the register class every later use names, so it stays there
-      asm volatile("" : "+" SDV2_Q_REG(qf[qb][ks]));
+      // with Q in AGPRs: the value is (re)defined in the register class every later
+      // use names, so it is never copied back and forth
+      if constexpr (kQB == 1) asm volatile("" : "+" SDV2_Q_REG(qf[qb][ks]));
     }
   }
 
