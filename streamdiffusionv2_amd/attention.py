@@ -38,12 +38,17 @@ _HOST_LIST_CACHE: dict = {}
 def _host_ints(value, slot: str, rows: Optional[int] = None) -> List[int]:
     """``current_start`` / ``grid_sizes`` as python ints.  A device tensor costs
     one copy per distinct (tensor, version): the same tensor is handed to every
-    layer of a forward, so all but the first layer hit the one-entry cache."""
+    layer of a forward, so all but the first layer hit the one-entry cache.  A
+    tensor without a version counter (created under ``torch.inference_mode()``)
+    may have been rewritten in place unnoticed - the reference shifts its
+    ``kv_cache_starts`` that way (causal_stream_inference.py:268-269) - and is
+    read every time."""
     if isinstance(value, torch.Tensor):
-        if value.device.type == "cpu":
+        version = ring.tensor_version(value)
+        if value.device.type == "cpu" or version is None:
             out = value.reshape(-1).tolist()
         else:
-            stamp = (value._version, value.data_ptr(), tuple(value.shape))
+            stamp = (version, value.data_ptr(), tuple(value.shape))
             hit = _HOST_LIST_CACHE.get(slot)
             if hit is not None and hit[0] is value and hit[1] == stamp:
                 out = hit[2]

@@ -59,7 +59,11 @@ _FREQS_CACHE: dict = {}
 def device_freqs(freqs: torch.Tensor, device: torch.device) -> torch.Tensor:
     """The complex128 [rows, 64] RoPE table as float64 [rows, 64, 2] on
     ``device``.  Converted once per (table, device)."""
-    key = (id(freqs), freqs._version, freqs.data_ptr(), str(device))
+    try:
+        version = freqs._version
+    except RuntimeError:            # created under torch.inference_mode(): no edit counter
+        version = None
+    key = (id(freqs), version, freqs.data_ptr(), str(device))
     hit = _FREQS_CACHE.get(key)
     if hit is not None and hit[0] is freqs:
         return hit[1]

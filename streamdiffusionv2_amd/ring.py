@@ -13,7 +13,9 @@ integers only.  The reference reads the two index tensors back with ``.item()``
 for every row of every layer; here the host carries a mirror of them (they are
 a pure function of the host-known ``current_start`` sequence), validated
 against the tensors' identity and version counter, so the steady state issues
-no device-to-host copy at all.  The kernel stores the new index values, which
+no device-to-host copy at all.  Tensors created under ``torch.inference_mode()``
+keep no version counter: for those only the identity is checked, and code that
+rewrites the two index tensors in place must call :func:`forget_index_mirror`.  The kernel stores the new index values, which
 keeps the tensors authoritative for every external consumer of the dict.
 """
 from __future__ import annotations
@@ -25,6 +27,16 @@ import torch
 
 HEAD_DIM = 128
 _MIRROR_KEY = "_sdv2_host_index_mirror"
+
+
+def tensor_version(t: torch.Tensor) -> Optional[int]:
+    """The tensor's in-place edit counter, or None for a tensor created under
+    ``torch.inference_mode()`` (the reference's API level runs in it,
+    streamdiffusionv2/pipeline.py:281,361), which keeps none."""
+    try:
+        return t._version
+    except RuntimeError:
+        return None
 
 
 def new_kv_cache(
@@ -103,8 +115,8 @@ def expand_crossattn_for_stream_batch(crossattn_cache: List[dict], batch_size: i
 class _IndexMirror:
     g_tensor: torch.Tensor
     l_tensor: torch.Tensor
-    g_version: int
-    l_version: int
+    g_version: Optional[int]
+    l_version: Optional[int]
     global_end: List[int]
     local_end: List[int]
 
@@ -112,7 +124,7 @@ class _IndexMirror:
         g, l = kv_cache["global_end_index"], kv_cache["local_end_index"]
         return (
             g is self.g_tensor and l is self.l_tensor
-            and g._version == self.g_version and l._version == self.l_version
+            and tensor_version(g) == self.g_version and tensor_version(l) == self.l_version
         )
 
 
@@ -120,7 +132,8 @@ def _mirror(kv_cache: dict) -> _IndexMirror:
     m: Optional[_IndexMirror] = kv_cache.get(_MIRROR_KEY)
     if m is None or not m.valid_for(kv_cache):
         g, l = kv_cache["global_end_index"], kv_cache["local_end_index"]
-        m = _IndexMirror(g, l, g._version, l._version, [int(x) for x in g.tolist()], [int(x) for x in l.tolist()])
+        m = _IndexMirror(g, l, tensor_version(g), tensor_version(l), [int(x) for x in g.tolist()],
+                         [int(x) for x in l.tolist()])
         kv_cache[_MIRROR_KEY] = m
     return m
 

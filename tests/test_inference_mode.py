@@ -1,0 +1,83 @@
+"""The reference runs its pipelines under ``torch.inference_mode()``
+(streamdiffusionv2/pipeline.py:281,361).  Tensors created there keep no
+in-place edit counter, which the host-side caches of this package otherwise
+use to notice edits; without it they must fall back to what is still safe.
+
+CPU: the ring planner on index tensors without a counter.  GPU: a stream run
+entirely under inference mode - caches allocated inside, ``current_start``
+handed over as one device tensor that is rewritten in place between calls, as
+the reference's ``kv_cache_starts`` is (causal_stream_inference.py:268-269) -
+against the oracle.
+"""
+import pytest
+import torch
+
+from oracle import sdv2_oracle as oracle
+
+
+def test_planner_on_tensors_without_a_version_counter():
+    from streamdiffusionv2_amd import ring
+
+    with torch.inference_mode():
+        cache = {"k": torch.zeros(1, 18, 1, 128), "v": torch.zeros(1, 18, 1, 128),
+                 "global_end_index": torch.zeros(1, dtype=torch.long),
+                 "local_end_index": torch.zeros(1, dtype=torch.long), "total_steps": 1, "current_step": 1}
+        with pytest.raises(RuntimeError):
+            cache["k"]._version                    # the premise of this test
+        assert ring.tensor_version(cache["k"]) is None
+        queue = [[]]
+        slots = [ring.plan_append(cache, queue, [c * 6], 6, 6, 1).dst_start[0] for c in range(6)]
+        assert slots == [0, 6, 12, 6, 12, 6]
+        # an in-place rewrite goes unnoticed by design; forgetting the mirror re-reads the tensors
+        cache["local_end_index"].fill_(6)
+        cache["global_end_index"].fill_(6)
+        stale = ring.plan_append(cache, [[12, 18]], [6], 6, 6, 1)
+        assert stale.new_local_end == [18]         # still the mirror's "cache is full" view: evicts
+        cache["local_end_index"].fill_(6)
+        cache["global_end_index"].fill_(6)
+        ring.forget_index_mirror(cache)
+        plan = ring.plan_append(cache, [[]], [6], 6, 6, 1)
+        assert plan.dst_start == [6] and plan.new_local_end == [12]
+    assert ring.tensor_version(torch.zeros(1)) == 0
+
+
+@pytest.mark.gpu
+def test_stream_under_inference_mode(gpu_device):
+    from streamdiffusionv2_amd import ring, rope
+    from streamdiffusionv2_amd.attention import RingKVPath
+
+    print("stream under torch.inference_mode()", flush=True)
+    heads, grid, cap_frames, rows = 2, (1, 4, 6), 4, 2
+    S = 24
+    freqs = rope.build_freqs()
+    o_cache = oracle.new_kv_cache(1, 1, cap_frames * S, heads, 1)[0]
+    o_path = oracle.RingAttentionOracle(sink_size=1)
+    gen = torch.Generator().manual_seed(3)
+    with torch.inference_mode():
+        cache = ring.new_kv_cache(1, 1, cap_frames * S, heads, 1, device=gpu_device)[0]
+        path = RingKVPath(sink_size=1)
+        starts_dev = torch.zeros(rows, dtype=torch.long, device=gpu_device)
+        grid_dev = torch.tensor([grid] * rows, device=gpu_device)
+        for call in range(9):
+            if call == 1:
+                ring.replicate_for_stream_batch([cache], rows)
+                oracle.replicate_for_stream_batch([o_cache], rows)
+            n = 1 if call == 0 else rows
+            starts = [max(call - r, 0) * S for r in range(n)]
+            # the same tensor object every call, rewritten in place
+            starts_dev[1:] = starts_dev[:-1].clone()
+            starts_dev[0] = call * S
+            assert starts_dev.tolist()[:n] == starts
+            q, k, v = (torch.randn(n, S, heads, 128, generator=gen).bfloat16() for _ in range(3))
+            got = path.attend(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), grid_dev[:n], freqs, cache,
+                              starts_dev[:n] if n < rows else starts_dev)
+            _, want_q, seq = o_path.step(q, k, v, [list(grid)] * n, freqs, o_cache, starts, with_attention=False)
+            torch.cuda.synchronize()
+            assert path.evict_idx == o_path.evict_idx, call
+            for name in ("global_end_index", "local_end_index"):
+                assert cache[name].tolist() == o_cache[name].tolist(), (call, name)
+            for name in ("k", "v"):
+                assert torch.equal(cache[name].cpu().view(torch.int16), o_cache[name].view(torch.int16)), (call, name)
+            want = oracle.attention_fp32_reference(want_q, o_cache["k"], o_cache["v"], seq)
+            err = (got.float().cpu() - want).abs()
+            assert err.max().item() <= 2e-2 and err.mean().item() <= 2e-3
