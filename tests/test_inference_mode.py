@@ -81,3 +81,75 @@ def test_stream_under_inference_mode(gpu_device):
             want = oracle.attention_fp32_reference(want_q, o_cache["k"], o_cache["v"], seq)
             err = (got.float().cpu() - want).abs()
             assert err.max().item() <= 2e-2 and err.mean().item() <= 2e-3
+
+
+@pytest.mark.gpu
+def test_rope_table_handed_over_on_the_device(gpu_device):
+    """The reference moves ``self.freqs`` to the activations' device inside the
+    forward (causal_model.py:253-266 reads it there), so the table arrives as
+    a complex128 CUDA tensor; the result must be the CPU table's."""
+    from streamdiffusionv2_amd import ops, rope
+
+    freqs = rope.build_freqs()
+    with torch.inference_mode():
+        on_device = freqs.to(gpu_device)
+        a = ops.device_freqs(freqs, gpu_device)
+        b = ops.device_freqs(on_device, gpu_device)
+        assert b.device == gpu_device and b.dtype == torch.float64 and tuple(b.shape) == (1024, 64, 2)
+        assert torch.equal(a, b)
+        assert ops.device_freqs(on_device, gpu_device) is b        # converted once
+
+
+@pytest.mark.gpu
+def test_module_called_the_way_the_reference_calls_it(gpu_device):
+    """CausalWanAttentionBlock.forward's call (causal_model.py:463-467) with what
+    the reference hands over: a cache dict built as _initialize_kv_cache builds it
+    (token-major zeros, causal_stream_inference.py:98-105), grid_sizes,
+    current_start and current_end as device tensors, freqs on the device, all
+    under inference mode.  Expected output: the module's own projections in
+    torch around the oracle's path."""
+    from streamdiffusionv2_amd import rope
+    from streamdiffusionv2_amd.attention import CausalWanSelfAttention
+
+    print("module seam, reference-style arguments", flush=True)
+    torch.manual_seed(5)
+    dim, heads, grid = 256, 2, (1, 4, 6)
+    S, cap = 24, 72
+    mod = CausalWanSelfAttention(dim, heads).to(gpu_device).bfloat16()
+    mod.sink_size = 1
+    with torch.no_grad():
+        mod.norm_q.weight.uniform_(0.5, 1.5)
+        mod.norm_k.weight.uniform_(0.5, 1.5)
+    o_cache = oracle.new_kv_cache(1, 1, cap, heads, 1)[0]
+    o_path = oracle.RingAttentionOracle(sink_size=1)
+    with torch.inference_mode():
+        freqs = rope.build_freqs().to(gpu_device)
+        kv_cache = {
+            "k": torch.zeros([1, cap, heads, 128], dtype=torch.bfloat16, device=gpu_device),
+            "v": torch.zeros([1, cap, heads, 128], dtype=torch.bfloat16, device=gpu_device),
+            "global_end_index": torch.tensor([0], dtype=torch.long, device=gpu_device),
+            "local_end_index": torch.tensor([0], dtype=torch.long, device=gpu_device),
+            "total_steps": 1, "current_step": 1,
+        }
+        grid_sizes = torch.tensor([grid], dtype=torch.long, device=gpu_device)
+        for call in range(6):
+            x = torch.randn(1, S, dim, device=gpu_device).bfloat16()
+            start = torch.tensor([call * S], dtype=torch.long, device=gpu_device)
+            end = torch.tensor([(call + 1) * S], dtype=torch.long, device=gpu_device)
+            y = mod(x, None, grid_sizes, freqs, None, kv_cache=kv_cache, current_start=start, current_end=end)
+            q = mod.norm_q(mod.q(x)).view(1, S, heads, 128).cpu()
+            k = mod.norm_k(mod.k(x)).view(1, S, heads, 128).cpu()
+            v = mod.v(x).view(1, S, heads, 128).cpu()
+            _, want_q, seq = o_path.step(q, k, v, [list(grid)], oracle.build_freqs(), o_cache, [call * S],
+                                         with_attention=False)
+            attn = oracle.attention_fp32_reference(want_q, o_cache["k"], o_cache["v"], seq)
+            want = mod.o(attn.to(gpu_device).bfloat16().flatten(2)).float().cpu()
+            torch.cuda.synchronize()
+            assert tuple(y.shape) == (1, S, dim) and y.dtype == torch.bfloat16
+            for name in ("k", "v"):
+                assert torch.equal(kv_cache[name].cpu().view(torch.int16), o_cache[name].view(torch.int16)), (call, name)
+            for name in ("global_end_index", "local_end_index"):
+                assert kv_cache[name].tolist() == o_cache[name].tolist(), (call, name)
+            assert mod.evict_idx == o_path.evict_idx
+            scale = max(1.0, want.abs().max().item())
+            assert (y.float().cpu() - want).abs().max().item() <= 3e-2 * scale, call
