@@ -56,6 +56,8 @@ def parse_args():
     ap.add_argument("--zero-inputs", action="store_true",
                     help="all-zero q/k/v and caches: nothing toggles, the chip holds its top clock (a diagnostic of "
                          "how much of the distance to the roofline is power, never a result)")
+    ap.add_argument("--torch-reference", action="store_true",
+                    help="also time the reference's op sequence in stock PyTorch on this GPU (its path without flash_attn)")
     ap.add_argument("--adaptive-sink", action="store_true",
                     help="also time the stream with the adaptive sink refresh on (one-frame chunks, one row)")
     ap.add_argument("--handoff", action="store_true",
@@ -285,6 +287,75 @@ def qk_norm_section(args, w):
     return out
 
 
+def torch_reference_section(args, w, ours_ms_per_step):
+    """The reference's op sequence for this path in stock PyTorch on the same
+    GPU - what models/wan/causal_model.py executes on a box without flash_attn:
+    RoPE of q and k as a complex128 multiply (:94-108), the two slice writes
+    into the token-major cache (:321-322), the index fills (:339-342) and
+    F.scaled_dot_product_attention on the cache view (:111-137).  Restated here
+    with every benefit of the doubt: expanded RoPE factors prepared once (its
+    rope cache), no ``.item()`` read-backs, steady-state slot rotation on host
+    integers.  A few layers are timed and scaled to the layer count."""
+    import torch.nn.functional as F
+
+    dev = torch.device("cuda:0")
+    from streamdiffusionv2_amd import workloads
+
+    B, S, H, L = w.rows, w.chunk_tokens, w.heads, w.cache_tokens
+    layers = min(w.layers, 4)
+    f, h, ww = w.grid
+    freqs = build_freqs()
+    c = freqs.shape[1]
+    parts = freqs.split([c - 2 * (c // 3), c // 3, c // 3], dim=1)
+    factors = torch.cat([parts[0][5:5 + f].view(f, 1, 1, -1).expand(f, h, ww, -1),
+                         parts[1][:h].view(1, h, 1, -1).expand(f, h, ww, -1),
+                         parts[2][:ww].view(1, 1, ww, -1).expand(f, h, ww, -1)], dim=-1).reshape(S, 1, -1).to(dev)
+    caches = [{"k": torch.randn(B, L, H, 128, device=dev).bfloat16() * w.input_scale,
+               "v": torch.randn(B, L, H, 128, device=dev).bfloat16() * w.input_scale,
+               "global_end_index": torch.zeros(B, dtype=torch.long, device=dev),
+               "local_end_index": torch.zeros(B, dtype=torch.long, device=dev)} for _ in range(layers)]
+    qkv = [tuple(t.to(dev) for t in workloads.make_qkv(w, 0, layer)) for layer in range(layers)]
+    slots = (L - S) // S                       # rotating slots behind the first chunk
+
+    def rope(x):
+        out = x.clone()
+        for i in range(B):
+            xi = torch.view_as_complex(x[i].to(torch.float64).reshape(S, H, -1, 2))
+            out[i] = torch.view_as_real(xi * factors).flatten(2).type_as(x)
+        return out
+
+    def layer_call(layer, call):
+        q, k, v = qkv[layer]
+        cache = caches[layer]
+        rq, rk = rope(q), rope(k)
+        end = S + (call % slots + 1) * S
+        for i in range(B):
+            cache["k"][i, end - S:end] = rk[i]
+            cache["v"][i, end - S:end] = v[i]
+            cache["global_end_index"][i].fill_(call * S)
+            cache["local_end_index"][i].fill_(L)
+        x = F.scaled_dot_product_attention(rq.transpose(1, 2), cache["k"].transpose(1, 2), cache["v"].transpose(1, 2),
+                                           attn_mask=None, dropout_p=0.0, is_causal=False)
+        return x.transpose(1, 2).contiguous()
+
+    for call in range(2):
+        for layer in range(layers):
+            layer_call(layer, call)
+    torch.cuda.synchronize()
+    steps = 3
+    t0 = time.perf_counter()
+    for call in range(2, 2 + steps):
+        for layer in range(layers):
+            layer_call(layer, call)
+    torch.cuda.synchronize()
+    per_layer_ms = (time.perf_counter() - t0) * 1e3 / (steps * layers)
+    ms_per_step = per_layer_ms * w.layers
+    return {"ms_per_step": ms_per_step, "tokens_per_s": B * S / (ms_per_step * 1e-3), "layers_timed": layers,
+            "speedup_of_this_library": ms_per_step / ours_ms_per_step,
+            "what": "reference op sequence in stock PyTorch on this GPU (complex128 RoPE, slice writes, SDPA); "
+                    f"torch {torch.__version__}"}
+
+
 def adaptive_sink_section(args, w):
     """Steady-state chunks with the adaptive sink refresh on (sink 3, threshold
     0.2: configs/wan_causal_dmd_v2v.yaml:55-56) against the same stream with it
@@ -498,6 +569,8 @@ def main():
         result["handoff"] = handoff_section(args, w)
     if args.adaptive_sink:
         result["adaptive_sink"] = adaptive_sink_section(args, w)
+    if args.torch_reference:
+        result["torch_gpu_reference"] = torch_reference_section(args, w, g["ms_per_step"])
     if not args.skip_mfma_reference:
         ref = mfma_reference()
         ref["attention_vs_random"] = achieved_tflops / ref["random"]
