@@ -350,7 +350,20 @@ def torch_reference_section(args, w, ours_ms_per_step):
     torch.cuda.synchronize()
     per_layer_ms = (time.perf_counter() - t0) * 1e3 / (steps * layers)
     ms_per_step = per_layer_ms * w.layers
-    return {"ms_per_step": ms_per_step, "tokens_per_s": B * S / (ms_per_step * 1e-3), "layers_timed": layers,
+    # its attention operator alone, on the same views
+    rq = rope(qkv[0][0]).transpose(1, 2)
+    kt, vt = caches[0]["k"].transpose(1, 2), caches[0]["v"].transpose(1, 2)
+    for _ in range(2):
+        F.scaled_dot_product_attention(rq, kt, vt)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(5):
+        F.scaled_dot_product_attention(rq, kt, vt)
+    e1.record()
+    torch.cuda.synchronize()
+    sdpa_ms = e0.elapsed_time(e1) / 5
+    return {"ms_per_step": ms_per_step, "sdpa_ms_per_layer": sdpa_ms,
+            "sdpa_TFLOPs": w.attn_flops() / (sdpa_ms * 1e-3) / 1e12, "tokens_per_s": B * S / (ms_per_step * 1e-3), "layers_timed": layers,
             "speedup_of_this_library": ms_per_step / ours_ms_per_step,
             "what": "reference op sequence in stock PyTorch on this GPU (complex128 RoPE, slice writes, SDPA); "
                     f"torch {torch.__version__}"}
