@@ -58,6 +58,21 @@ def build(verbose: bool = False, keep_temps: bool = False) -> Path:
     return LIB_PATH
 
 
+GPU_CALLER_SRC = REPO_ROOT / "tests" / "c_abi" / "gpu_caller.cpp"
+GPU_CALLER_BIN = REPO_ROOT / "tests" / "c_abi" / "_bin" / "gpu_caller"
+
+
+def build_gpu_caller(verbose: bool = False) -> Path:
+    """The stand-alone C++ program of the GPU test suite that drives the
+    library through include/sdv2kv.h with nothing but the HIP runtime; built
+    here so that a GPU box only has to run it."""
+    GPU_CALLER_BIN.parent.mkdir(exist_ok=True)
+    _run([hipcc_path(), "-O2", "-std=c++17", "-Wno-unused-command-line-argument", "-Wno-unused-result",
+          f"-I{REPO_ROOT / 'include'}", str(GPU_CALLER_SRC), "-o", str(GPU_CALLER_BIN), f"-L{LIB_DIR}", "-lsdv2kv",
+          "-Wl,-rpath,$ORIGIN/../../../streamdiffusionv2_amd/_lib"], verbose)
+    return GPU_CALLER_BIN
+
+
 def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
@@ -72,3 +87,4 @@ def _run(cmd, verbose):
 
 if __name__ == "__main__":
     print(build(verbose=True, keep_temps="--keep-temps" in sys.argv))
+    print(build_gpu_caller(verbose=True))

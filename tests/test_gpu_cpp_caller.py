@@ -1,0 +1,73 @@
+"""The C ABI driven by a program that is not Python: tests/c_abi/gpu_caller.cpp
+(built by the package's build step) allocates with the HIP runtime, makes its
+own stream and runs append + attention chunk by chunk through
+include/sdv2kv.h.  Inputs go in and results come back through files; the
+expected values are the oracle's.  Nothing of PyTorch is in that process, so
+this is also the check that the library stands on the HIP runtime alone."""
+import os
+import struct
+import subprocess
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import sdv2_oracle as oracle
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CALLER = os.path.join(HERE, "c_abi", "_bin", "gpu_caller")
+
+
+def _bf16_bytes(t):
+    return t.contiguous().view(torch.int16).numpy().tobytes()
+
+
+def _bf16_from(buf, shape):
+    return torch.from_numpy(np.frombuffer(buf, dtype=np.int16).copy()).view(torch.bfloat16).reshape(shape)
+
+
+@pytest.mark.parametrize("splits", [1, 2])
+def test_cpp_program_runs_a_stream(gpu_device, tmp_path, splits):
+    assert os.path.exists(CALLER), f"{CALLER} is missing: build it with python -m streamdiffusionv2_amd.build_ext"
+    print(f"C++ caller, {splits} key range(s)", flush=True)
+    heads, grid, cap_frames, chunks = 3, (1, 5, 8), 3, 5
+    S = grid[1] * grid[2]
+    cap = cap_frames * S
+    gen = torch.Generator().manual_seed(21 + splits)
+    freqs = oracle.build_freqs()
+    o_cache = oracle.new_kv_cache(1, 1, cap, heads, 1)[0]
+    o_path = oracle.RingAttentionOracle(sink_size=1)
+
+    table = torch.view_as_real(freqs).contiguous().numpy().astype(np.float64)
+    blob = [struct.pack("<9i", chunks, S, heads, *grid, cap, table.shape[0], splits), table.tobytes()]
+    want = []
+    for c in range(chunks):
+        q, k, v = (torch.randn(1, S, heads, 128, generator=gen).bfloat16() for _ in range(3))
+        _, roped_q, seq = o_path.step(q, k, v, [list(grid)], freqs, o_cache, [c * S], with_attention=False)
+        (a, b), = o_path.last_writes
+        blob.append(struct.pack("<4q", c * S // S, a, o_cache["global_end_index"].item(), seq[0]))
+        blob += [_bf16_bytes(q), _bf16_bytes(k), _bf16_bytes(v)]
+        want.append((roped_q, oracle.attention_fp32_reference(roped_q, o_cache["k"], o_cache["v"], seq)))
+    (tmp_path / "in.bin").write_bytes(b"".join(blob))
+
+    run = subprocess.run([CALLER, str(tmp_path / "in.bin"), str(tmp_path / "out.bin")], capture_output=True, text=True,
+                         timeout=120)
+    assert run.returncode == 0, run.stdout + run.stderr
+    out = (tmp_path / "out.bin").read_bytes()
+    n = S * heads * 128 * 2
+    for c, (roped_q, attn) in enumerate(want):
+        got_q = _bf16_from(out[2 * c * n:(2 * c + 1) * n], (1, S, heads, 128))
+        got_o = _bf16_from(out[(2 * c + 1) * n:(2 * c + 2) * n], (1, S, heads, 128))
+        assert torch.equal(got_q.view(torch.int16), roped_q.view(torch.int16)), c
+        err = (got_o.float() - attn).abs()
+        assert err.max().item() <= 2e-2 and err.mean().item() <= 2e-3, c
+    off = 2 * chunks * n
+    nc = cap * heads * 128 * 2
+    for name in ("k", "v"):
+        got = _bf16_from(out[off:off + nc], (1, heads, cap, 128)).permute(0, 2, 1, 3)
+        assert torch.equal(got.contiguous().view(torch.int16), o_cache[name].view(torch.int16)), name
+        off += nc
+    g_end, l_end = struct.unpack("<2q", out[off:off + 16])
+    assert [g_end] == o_cache["global_end_index"].tolist() and [l_end] == o_cache["local_end_index"].tolist()
