@@ -33,6 +33,11 @@ moved_blocks_by_donor      streamv2v/communication/kv_cache_manager.py:126-136
 receive_kv_block           streamv2v/communication/kv_cache_manager.py:66-82
 =========================  ====================================================
 
+``oracle/rope_ring_ref.c`` restates ``causal_rope_apply`` (with the table
+expansion) and the placement state machine once more, in plain C without any
+shared code; ``tests/test_oracle_c_ref.py`` requires the two to agree bit for
+bit and checks the C side on its own against the hand traces.
+
 Pinning (what fixes each function independently of this file) lives in
 ``tests/test_oracle_*.py`` (and, for the four functions at the end of the
 table, in ``tests/test_fused_qk_norm.py``, ``tests/test_block_mask.py``,
