@@ -146,3 +146,19 @@ def test_plain_c_caller(tmp_path):
     assert run.returncode == 0, run.stdout + run.stderr
     assert "all checks passed" in run.stdout
     assert "splits for 1x1560 tokens, 12 heads, 9360 keys: 3" in run.stdout
+
+
+def test_documented_ctypes_struct_matches_the_binding():
+    """INTEGRATION.md shows a ctypes mirror of sdv2_attn_params for callers who
+    bind the library themselves; its field list must be the one the package's
+    own binding uses (a missing field shifts every later one)."""
+    import re
+
+    from streamdiffusionv2_amd import _capi
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    text = open(os.path.join(root, "INTEGRATION.md")).read()
+    block = text[text.index("class AttnParams(C.Structure):"):]
+    block = block[:block.index("p = AttnParams(")]
+    documented = re.findall(r'\("(\w+)",', block)
+    assert documented == [name for name, _ in _capi.AttnParams._fields_]
