@@ -2,6 +2,7 @@
  * (not C++), that the library links from C, and that argument validation
  * answers with status codes before anything touches a GPU.  Built and run by
  * tests/test_capi_symbols.py; prints one line per check. */
+#include <stddef.h>
 #include <stdio.h>
 #include <string.h>
 
@@ -64,6 +65,16 @@ int main(void) {
   rl.tokens = 0;
   rl.dst_global_end_index = (int64_t*)&rl;          /* destination index without a source */
   expect("relayout index without source", sdv2_cache_relayout(&rl), SDV2_ERR_INVALID_ARG);
+
+  /* struct layouts, for the bindings to compare themselves with */
+  printf("layout sdv2_append_params size=%zu stream=%zu dst_start_override=%zu\n", sizeof(sdv2_append_params),
+         offsetof(sdv2_append_params, stream), offsetof(sdv2_append_params, dst_start_override));
+  printf("layout sdv2_attn_params size=%zu stream=%zu chunk_key_start=%zu\n", sizeof(sdv2_attn_params),
+         offsetof(sdv2_attn_params, stream), offsetof(sdv2_attn_params, chunk_key_start));
+  printf("layout sdv2_sink_sim_params size=%zu stream=%zu override_rows=%zu\n", sizeof(sdv2_sink_sim_params),
+         offsetof(sdv2_sink_sim_params, stream), offsetof(sdv2_sink_sim_params, override_rows));
+  printf("layout sdv2_relayout_params size=%zu stream=%zu timing_stop=%zu\n", sizeof(sdv2_relayout_params),
+         offsetof(sdv2_relayout_params, stream), offsetof(sdv2_relayout_params, timing_stop));
 
   printf("splits for 1x1560 tokens, 12 heads, 9360 keys: %d\n", sdv2_swa_attn_default_splits(1, 1560, 12, 9360));
   printf("workspace for that call: %zu bytes\n", sdv2_swa_attn_workspace_bytes(1, 1560, 12, 9360, 0));

@@ -146,6 +146,17 @@ def test_plain_c_caller(tmp_path):
     assert run.returncode == 0, run.stdout + run.stderr
     assert "all checks passed" in run.stdout
     assert "splits for 1x1560 tokens, 12 heads, 9360 keys: 3" in run.stdout
+    # the ctypes structures must have the C compiler's layout
+    import ctypes as C
+    import re
+
+    for c_name, binding, last in (("sdv2_append_params", _capi.AppendParams, "dst_start_override"),
+                                  ("sdv2_attn_params", _capi.AttnParams, "chunk_key_start"),
+                                  ("sdv2_sink_sim_params", _capi.SinkSimParams, "override_rows"),
+                                  ("sdv2_relayout_params", _capi.RelayoutParams, "timing_stop")):
+        m = re.search(rf"layout {c_name} size=(\d+) stream=(\d+) {last}=(\d+)", run.stdout)
+        assert m, run.stdout
+        assert (C.sizeof(binding), binding.stream.offset, getattr(binding, last).offset) == tuple(map(int, m.groups())), c_name
 
 
 def test_documented_ctypes_struct_matches_the_binding():
