@@ -160,9 +160,9 @@ def test_plain_c_caller(tmp_path):
 
 
 def test_documented_ctypes_struct_matches_the_binding():
-    """INTEGRATION.md shows a ctypes mirror of sdv2_attn_params for callers who
-    bind the library themselves; its field list must be the one the package's
-    own binding uses (a missing field shifts every later one)."""
+    """The integration guide shows a ctypes mirror of sdv2_attn_params for
+    callers who bind the library themselves; its field list must be the one the
+    package's own binding uses (a missing field shifts every later one)."""
     import re
 
     from streamdiffusionv2_amd import _capi
