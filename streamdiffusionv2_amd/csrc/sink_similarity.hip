@@ -42,7 +42,7 @@ struct SinkSimKernelArgs {
   const void* v_cache;
   sdv2_stride3 k_in_st, v_in_st, k_st, v_st;
   const double2* freqs;
-  float* sums;                              // [rows][2*sink+2][kTokenSplits][heads*128]: token sums
+  float* sums;                              // [rows][2*sink+2][heads*128][kTokenSplits]: token sums
   float* similarity;                        // [rows][sink]
   int32_t* refresh;                         // [rows]
   int64_t* dst_override;                    // [rows] or null: slot start for the append that follows
@@ -144,8 +144,9 @@ void sink_frame_sum_kernel(const SinkSimKernelArgs a) {
 #pragma unroll
     for (int j = 0; j < kTokenLanes; ++j) s += part[j][threadIdx.x];
     const int64_t width = static_cast<int64_t>(a.heads) * 128;
-    a.sums[((static_cast<int64_t>(row) * (2 * sink + 2) + m) * kTokenSplits + split) * width + head * 128 +
-           threadIdx.x] = s;
+    // the token ranges of one column sit side by side, so the decision kernel fetches them with two 16-byte loads
+    a.sums[((static_cast<int64_t>(row) * (2 * sink + 2) + m) * width + head * 128 + threadIdx.x) * kTokenSplits +
+           split] = s;
   }
 }
 
@@ -179,16 +180,17 @@ void sink_decide_kernel(const SinkSimKernelArgs a) {
   // means of frame m at this thread's columns: the token ranges in order, then the rounding of a stored mean
   auto means = [&](int m, float (&out)[kCols]) {
     const float* p = sums + static_cast<int64_t>(m) * kTokenSplits * width;
-    float part[kCols][kTokenSplits];
+    float4 part[kCols][kTokenSplits / 4];
 #pragma unroll
     for (int i = 0; i < kCols; ++i)
 #pragma unroll
-      for (int j = 0; j < kTokenSplits; ++j) part[i][j] = p[static_cast<int64_t>(j) * width + col[i]];
+      for (int j = 0; j < kTokenSplits / 4; ++j)
+        part[i][j] = *reinterpret_cast<const float4*>(p + static_cast<int64_t>(col[i]) * kTokenSplits + 4 * j);
 #pragma unroll
     for (int i = 0; i < kCols; ++i) {
       float s = 0.f;
 #pragma unroll
-      for (int j = 0; j < kTokenSplits; ++j) s += part[i][j];
+      for (int j = 0; j < kTokenSplits / 4; ++j) s = (((s + part[i][j].x) + part[i][j].y) + part[i][j].z) + part[i][j].w;
       out[i] = round_to_storage<T>(s * inv_tokens) * live[i];
     }
   };
