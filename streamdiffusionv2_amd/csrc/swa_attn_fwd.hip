@@ -59,6 +59,8 @@ typedef __attribute__((ext_vector_type(2))) float f32x2;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((address_space(3))) char lds_char;
 
 constexpr int kD = SDV2_HEAD_DIM;           // 128
@@ -111,8 +113,9 @@ struct AttnKernelArgs {
   float scale_log2;            // softmax_scale * log2(e)
   int32_t mask_block_tokens;   // 0 = no mask inside the chunk
   const int32_t* chunk_start;  // device [rows]: cache position of the chunk's own first key
-  float* part_o;               // [split][row][head][q][128] fp32, normalised
+  uint16_t* part_o;            // [split][row][head][q][128] fp16: normalised output / row scale
   float* part_lse;             // [split][row][head][q]      log2 sum exp
+  float* part_scale;           // [split][row][head][q]      largest magnitude of the normalised row
 };
 
 __device__ __forceinline__ int swz(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
@@ -138,6 +141,12 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
   // fptrunc <2 x float> -> <2 x bfloat> selects v_cvt_pk_bf16_f32 (nearest-even)
   const f32x2 x = {lo, hi};
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+}
+
+// two floats -> packed fp16 pair (lo in the low half), nearest-even
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+  const f32x2 x = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(x, f16x2));
 }
 
 // acc + lo + hi of a packed bf16 pair (v_dot2c_f32_bf16 against (1, 1))
@@ -789,9 +798,9 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   // A lane holds one query row's values scattered over the 128 dims, so direct
   // stores would touch 32 rows with 16 or 32 bytes each.  Instead every wave
   // stages one 32-row block at a time in its own 16 KB of the (now idle) LDS,
-  // 16-byte chunks XOR-swizzled by row, and writes whole rows: 256 bytes of bf16
-  // for the result of an unsplit call, 512 bytes of fp32 for the normalised
-  // partial result of a split call (plus its log-sum-exp).  LDS operations of
+  // 16-byte chunks XOR-swizzled by row, and writes whole rows of 256 bytes: bf16
+  // for the result of an unsplit call, scaled fp16 for the partial result of a
+  // split call (plus its scale and log-sum-exp).  LDS operations of
   // one wave complete in order, so the block needs no barrier of its own.
   __syncthreads();                    // every wave is done with the K / V buffers
   lds_char* stage = lds + wave * kStageBytes;
@@ -824,29 +833,42 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
         if (q0 + qb * 32 + rr < a.q_tokens) *reinterpret_cast<u32x4*>(dst + rr * a.o_st.token + j * 8) = w;
       }
     } else {
+      // Partial result of a key range: the normalised row divided by its largest
+      // magnitude, as fp16 (values in [-1, 1]: 11 bits against the row's scale,
+      // sixteen times finer than the bf16 of the final result), plus that scale
+      // and the log-sum-exp.  Half the bytes of an fp32 partial, written and read.
+      float amax = 0.f;
+#pragma unroll
+      for (int db = 0; db < 4; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) amax = vmax(amax, __builtin_fabsf(oacc[qb][db][i]));
+      amax = half_max(amax) * inv;
+      const float row_scale = amax > 0.f && amax < INFINITY ? amax : 1.0f;
+      const float to_unit = inv / row_scale;
 #pragma unroll
       for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          f32x4 w;
-          w[0] = oacc[qb][db][4 * g] * inv;
-          w[1] = oacc[qb][db][4 * g + 1] * inv;
-          w[2] = oacc[qb][db][4 * g + 2] * inv;
-          w[3] = oacc[qb][db][4 * g + 3] * inv;
-          const int chunk = db * 8 + 2 * g + hf;
-          *reinterpret_cast<__attribute__((address_space(3))) f32x4*>(stage + r * 512 + ((chunk ^ r) << 4)) = w;
+          u32x2 w;
+          w[0] = pack_f16x2(oacc[qb][db][4 * g] * to_unit, oacc[qb][db][4 * g + 1] * to_unit);
+          w[1] = pack_f16x2(oacc[qb][db][4 * g + 2] * to_unit, oacc[qb][db][4 * g + 3] * to_unit);
+          const int chunk = db * 4 + g;
+          *reinterpret_cast<__attribute__((address_space(3))) u32x2*>(
+              stage + r * 256 + ((chunk ^ (r & 15)) << 4) + hf * 8) = w;
         }
       const int64_t prow0 = (((int64_t)split * a.rows + row) * a.heads + head) * a.q_tokens + q0 + qb * 32;
-      if (hf == 0 && q_row[qb] < a.q_tokens)
+      if (hf == 0 && q_row[qb] < a.q_tokens) {
         a.part_lse[prow0 + r] = l_tot > 0.f ? m_run[qb] * c.c2 + __builtin_amdgcn_logf(l_tot) : -INFINITY;
-      float* dst = a.part_o + prow0 * kD;
-      const int j = lane & 31;
+        a.part_scale[prow0 + r] = row_scale;
+      }
+      uint16_t* dst = a.part_o + prow0 * kD;
+      const int j = lane & 15;
 #pragma unroll
-      for (int it = 0; it < 16; ++it) {
-        const int rr = 2 * it + (lane >> 5);
-        const f32x4 w = *reinterpret_cast<__attribute__((address_space(3))) const f32x4*>(
-            stage + rr * 512 + ((j ^ rr) << 4));
-        if (q0 + qb * 32 + rr < a.q_tokens) *reinterpret_cast<f32x4*>(dst + rr * kD + j * 4) = w;
+      for (int it = 0; it < 8; ++it) {
+        const int rr = 4 * it + (lane >> 4);
+        const u32x4 w = *reinterpret_cast<__attribute__((address_space(3))) const u32x4*>(
+            stage + rr * 256 + ((j ^ (rr & 15)) << 4));
+        if (q0 + qb * 32 + rr < a.q_tokens) *reinterpret_cast<u32x4*>(dst + rr * kD + j * 8) = w;
       }
     }
   }
@@ -872,10 +894,10 @@ void swa_attn_merge_kernel(const AttnKernelArgs a) {
     const float lse = a.part_lse[s * nq + idx];
     const float w = lse == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(lse - lse_max);
     wsum += w;
-    const float4* po = reinterpret_cast<const float4*>(a.part_o + (s * nq + idx) * kD + lane * 8);
-    const float4 x = po[0], y = po[1];
-    acc[0] += w * x.x; acc[1] += w * x.y; acc[2] += w * x.z; acc[3] += w * x.w;
-    acc[4] += w * y.x; acc[5] += w * y.y; acc[6] += w * y.z; acc[7] += w * y.w;
+    const float ws = w * a.part_scale[s * nq + idx];          // weight times the row's fp16 scale
+    const f16x8 x = *reinterpret_cast<const f16x8*>(a.part_o + (s * nq + idx) * kD + lane * 8);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] += ws * static_cast<float>(x[i]);
   }
   const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
   uint4 o;
@@ -899,12 +921,12 @@ extern "C" int sdv2_swa_attn_default_splits(int32_t rows, int32_t q_tokens, int3
   // One workgroup per CU.  With s key-range splits there are qwork * s
   // workgroups; they run in ceil(qwork * s / 256) rounds, each as long as one
   // workgroup's tile count plus a fixed start / end cost of about three tile
-  // times.  Writing and merging the fp32 partial
+  // times.  Writing and merging the fp16 partial
   // results costs roughly one tile time per 7 MB per split.  Constants fitted
   // to measurements on the five benchmark shapes.
   const int64_t qwork = (int64_t)rows * heads * ((q_tokens + kQTile - 1) / kQTile);
   const int ntiles = (max_seq_len + kKTile - 1) / kKTile;
-  const double partial_tiles = (double)rows * heads * q_tokens * kD * 4 / 7.0e6;
+  const double partial_tiles = (double)rows * heads * q_tokens * kD * 2 / 7.0e6;
   int best = 1;
   double best_cost = 1e300;
   for (int sp = 1; sp <= 8; ++sp) {
@@ -922,8 +944,8 @@ extern "C" size_t sdv2_swa_attn_workspace_bytes(int32_t rows, int32_t q_tokens, 
   if (num_splits <= 0) num_splits = sdv2_swa_attn_default_splits(rows, q_tokens, heads, max_seq_len);
   if (num_splits <= 1) return 0;
   const size_t nq = (size_t)rows * heads * q_tokens;
-  return align_up((size_t)num_splits * nq * kD * sizeof(float), 256) +
-         align_up((size_t)num_splits * nq * sizeof(float), 256);
+  return align_up((size_t)num_splits * nq * kD * sizeof(uint16_t), 256) +
+         2 * align_up((size_t)num_splits * nq * sizeof(float), 256);
 }
 
 extern "C" int sdv2_swa_attn_fwd(const sdv2_attn_params* p) {
@@ -972,9 +994,11 @@ extern "C" int sdv2_swa_attn_fwd(const sdv2_attn_params* p) {
     if (!p->workspace || p->workspace_bytes < need) return SDV2_ERR_WORKSPACE;
     if (reinterpret_cast<uintptr_t>(p->workspace) & 255) return SDV2_ERR_INVALID_ARG;
     const size_t nq = (size_t)p->rows * p->heads * p->q_tokens;
-    a.part_o = static_cast<float*>(p->workspace);
-    a.part_lse = reinterpret_cast<float*>(static_cast<char*>(p->workspace) +
-                                          align_up((size_t)splits * nq * kD * sizeof(float), 256));
+    char* ws = static_cast<char*>(p->workspace);
+    a.part_o = reinterpret_cast<uint16_t*>(ws);
+    ws += align_up((size_t)splits * nq * kD * sizeof(uint16_t), 256);
+    a.part_lse = reinterpret_cast<float*>(ws);
+    a.part_scale = reinterpret_cast<float*>(ws + align_up((size_t)splits * nq * sizeof(float), 256));
   }
 
   hipStream_t stream = static_cast<hipStream_t>(p->stream);
