@@ -31,9 +31,9 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # FETCH_SIZE and WRITE_SIZE counters (KiB per dispatch) on this same script and
 # scaled by what those counters read for a plain 256 MiB copy (x2.000 / x1.000).
 MEASURED_HBM_BYTES = {
-    "c2_wan1.3b_1560tok_6frames": {"attn": 99.68e6, "append": 29.09e6, "merge": 34.07e6, "splits": 3},
-    "c3_wan1.3b_b4_4680tok_12frames": {"attn": 1261.14e6, "append": 345.46e6, "merge": 408.43e6, "splits": 3},
-    "c5_720p_b2_10800tok_21frames": {"attn": 3840.53e6, "append": 398.98e6, "merge": 885.87e6, "splits": 6},
+    "c2_wan1.3b_1560tok_6frames": {"attn": 85.54e6, "append": 29.09e6, "merge": 20.14e6, "splits": 3},
+    "c3_wan1.3b_b4_4680tok_12frames": {"attn": 1071.13e6, "append": 345.47e6, "merge": 240.87e6, "splits": 3},
+    "c5_720p_b2_10800tok_21frames": {"attn": 3460.85e6, "append": 398.99e6, "merge": 566.36e6, "splits": 6},
 }
 
 
