@@ -55,7 +55,6 @@ statement: max-abs 2e-2, mean-abs 2e-3 against fp32).
 """
 from __future__ import annotations
 
-import math
 from typing import List, Optional, Sequence, Tuple
 
 import torch

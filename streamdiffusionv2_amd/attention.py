@@ -10,7 +10,7 @@ two HIP kernels and no device-to-host copy.
 """
 from __future__ import annotations
 
-from typing import List, Optional, Sequence, Tuple
+from typing import List, Optional
 
 import torch
 import torch.nn as nn

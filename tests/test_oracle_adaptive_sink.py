@@ -3,7 +3,6 @@ a hand trace of queue and writes with similarities that have closed forms, the
 similarity against a float64 numpy restatement of the definition, and the
 one-frame-chunk precondition."""
 import numpy as np
-import pytest
 import torch
 
 from oracle import sdv2_oracle as oracle
