@@ -32,6 +32,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # scaled by what those counters read for a plain 256 MiB copy (x2.000 / x1.000).
 MEASURED_HBM_BYTES = {
     "c2_wan1.3b_1560tok_6frames": {"attn": 85.54e6, "append": 29.09e6, "merge": 20.14e6, "splits": 3},
+    "c4_wan14b_1560tok_6frames": {"attn": 325.04e6, "append": 96.25e6, "merge": 84.02e6, "splits": 4},
     "c3_wan1.3b_b4_4680tok_12frames": {"attn": 1071.13e6, "append": 345.47e6, "merge": 240.87e6, "splits": 3},
     "c5_720p_b2_10800tok_21frames": {"attn": 3460.85e6, "append": 398.99e6, "merge": 566.36e6, "splits": 6},
 }

@@ -921,12 +921,12 @@ extern "C" int sdv2_swa_attn_default_splits(int32_t rows, int32_t q_tokens, int3
   // One workgroup per CU.  With s key-range splits there are qwork * s
   // workgroups; they run in ceil(qwork * s / 256) rounds, each as long as one
   // workgroup's tile count plus a fixed start / end cost of about three tile
-  // times.  Writing and merging the fp16 partial
-  // results costs roughly one tile time per 7 MB per split.  Constants fitted
+  // times.  Writing and merging the partial results
+  // costs roughly one tile time per 3.5 MB of them per split.  Constants fitted
   // to measurements on the five benchmark shapes.
   const int64_t qwork = (int64_t)rows * heads * ((q_tokens + kQTile - 1) / kQTile);
   const int ntiles = (max_seq_len + kKTile - 1) / kKTile;
-  const double partial_tiles = (double)rows * heads * q_tokens * kD * 2 / 7.0e6;
+  const double partial_tiles = (double)rows * heads * q_tokens * kD * 4 / 7.0e6;
   int best = 1;
   double best_cost = 1e300;
   for (int sp = 1; sp <= 8; ++sp) {
