@@ -86,10 +86,14 @@ const char* sdv2_status_string(int status);
  * decided by the caller's ring state machine (causal_model.py:302-342); the
  * kernel only performs the scatter and stores the two int64 indices, so
  * eviction costs nothing beyond the write of the new chunk.
+ *
+ * With k_in, v_in, k_cache and v_cache all NULL the call is the reference's
+ * causal_rope_apply on its own (causal_model.py:94-108): q_out = rope(q_in),
+ * no cache, index or dst_start is read or written.
  * ---------------------------------------------------------------------- */
 typedef struct sdv2_append_params {
   const void* q_in;            /* [B,S,H,128]; may be NULL together with q_out */
-  const void* k_in;
+  const void* k_in;            /* k_in, v_in and the caches: all or none       */
   const void* v_in;
   void* q_out;                 /* [B,S,H,128] roped query                      */
   void* k_cache;               /* [B,cap,H,128]                                */

@@ -63,7 +63,9 @@ __device__ __forceinline__ int64_t row_dst_start(const AppendKernelArgs& a, int 
   return dst;
 }
 
-template <typename T, bool kWithQ>
+// kWithKV = false: rotation of q alone (the stand-alone causal_rope_apply,
+// causal_model.py:94-108), no cache and no index is touched.
+template <typename T, bool kWithQ, bool kWithKV>
 __global__ __launch_bounds__(kLanesPerRow * kTokensPerBlock)
 void kv_append_rope_kernel(const AppendKernelArgs a) {
   const int lane = threadIdx.x & (kLanesPerRow - 1);
@@ -71,7 +73,7 @@ void kv_append_rope_kernel(const AppendKernelArgs a) {
   const int row = blockIdx.z;
   const int head0 = blockIdx.y * kHeadsPerThread;
 
-  if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+  if (kWithKV && blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
     if (a.global_end) a.global_end[row] = a.new_global[row];
     if (a.local_end) a.local_end[row] = a.new_local[row];
   }
@@ -87,7 +89,7 @@ void kv_append_rope_kernel(const AppendKernelArgs a) {
   sdv2::load_rotation(a.freqs, a.pairs, a.split_t, a.split_h, lane, frame, hi, wi, cs);
 
   const int64_t e0 = lane * 8;
-  const int64_t dst_tok = row_dst_start(a, row) + tok;
+  const int64_t dst_tok = kWithKV ? row_dst_start(a, row) + tok : 0;
   const T* qi = static_cast<const T*>(a.q_in) + row * a.q_in_st.row + tok * a.q_in_st.token + e0;
   const T* ki = static_cast<const T*>(a.k_in) + row * a.k_in_st.row + tok * a.k_in_st.token + e0;
   const T* vi = static_cast<const T*>(a.v_in) + row * a.v_in_st.row + tok * a.v_in_st.token + e0;
@@ -100,8 +102,10 @@ void kv_append_rope_kernel(const AppendKernelArgs a) {
   for (int j = 0; j < kHeadsPerThread; ++j) {
     const int h = head0 + j;
     if (h < a.heads) {
-      k[j] = sdv2::Vec8<T>::load(ki + h * a.k_in_st.head);
-      v[j] = sdv2::Vec8<T>::load(vi + h * a.v_in_st.head);
+      if (kWithKV) {
+        k[j] = sdv2::Vec8<T>::load(ki + h * a.k_in_st.head);
+        v[j] = sdv2::Vec8<T>::load(vi + h * a.v_in_st.head);
+      }
       if (kWithQ) q[j] = sdv2::Vec8<T>::load(qi + h * a.q_in_st.head);
     }
   }
@@ -109,8 +113,10 @@ void kv_append_rope_kernel(const AppendKernelArgs a) {
   for (int j = 0; j < kHeadsPerThread; ++j) {
     const int h = head0 + j;
     if (h < a.heads) {
-      v[j].store(vc + h * a.v_st.head);
-      sdv2::rotate(k[j], cs).store(kc + h * a.k_st.head);
+      if (kWithKV) {
+        v[j].store(vc + h * a.v_st.head);
+        sdv2::rotate(k[j], cs).store(kc + h * a.k_st.head);
+      }
       if (kWithQ) sdv2::rotate(q[j], cs).store(qo + h * a.q_out_st.head);
     }
   }
@@ -228,12 +234,20 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
   if (p->rows == 0 || p->tokens == 0) return SDV2_OK;
   if (p->grid_f <= 0 || p->grid_h <= 0 || p->grid_w <= 0) return SDV2_ERR_INVALID_ARG;
   if (static_cast<int64_t>(p->grid_f) * p->grid_h * p->grid_w != p->tokens) return SDV2_ERR_INVALID_ARG;
-  if (!p->k_in || !p->v_in || !p->k_cache || !p->v_cache || !p->freqs) return SDV2_ERR_INVALID_ARG;
+  if (!p->freqs) return SDV2_ERR_INVALID_ARG;
   if ((p->q_in == nullptr) != (p->q_out == nullptr)) return SDV2_ERR_INVALID_ARG;
-  if (!p->start_frame || !p->dst_start) return SDV2_ERR_INVALID_ARG;
+  const bool with_q = p->q_in != nullptr;
+  // k, v and the two caches come together or not at all; without them the call
+  // only rotates q (and then has nothing to do with a cache or its indices)
+  const bool with_kv = p->k_in != nullptr;
+  if ((p->v_in != nullptr) != with_kv || (p->k_cache != nullptr) != with_kv || (p->v_cache != nullptr) != with_kv)
+    return SDV2_ERR_INVALID_ARG;
+  if (!with_kv && (!with_q || p->global_end_index || p->local_end_index || p->dst_start_override ||
+                   p->q_norm_weight || p->k_norm_weight))
+    return SDV2_ERR_INVALID_ARG;
+  if (!p->start_frame || (with_kv && !p->dst_start)) return SDV2_ERR_INVALID_ARG;
   if ((p->global_end_index || p->local_end_index) && (!p->new_global_end || !p->new_local_end))
     return SDV2_ERR_INVALID_ARG;
-  const bool with_q = p->q_in != nullptr;
   if ((p->timing_start == nullptr) != (p->timing_stop == nullptr)) return SDV2_ERR_INVALID_ARG;
   const bool with_norm = p->q_norm_weight != nullptr || p->k_norm_weight != nullptr;
   if (with_norm) {
@@ -249,8 +263,8 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
   const void* ptrs[] = {p->q_in, p->k_in, p->v_in, p->q_out, p->k_cache, p->v_cache};
   for (const void* ptr : ptrs)
     if (ptr && !aligned16(ptr)) return SDV2_ERR_INVALID_ARG;
-  if (!stride_ok(p->k_in_stride, vec) || !stride_ok(p->v_in_stride, vec) ||
-      !stride_ok(p->k_cache_stride, vec) || !stride_ok(p->v_cache_stride, vec))
+  if (with_kv && (!stride_ok(p->k_in_stride, vec) || !stride_ok(p->v_in_stride, vec) ||
+                  !stride_ok(p->k_cache_stride, vec) || !stride_ok(p->v_cache_stride, vec)))
     return SDV2_ERR_INVALID_ARG;
   if (with_q && (!stride_ok(p->q_in_stride, vec) || !stride_ok(p->q_out_stride, vec)))
     return SDV2_ERR_INVALID_ARG;
@@ -258,7 +272,8 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
   if (p->grid_h > p->freq_rows || p->grid_w > p->freq_rows) return SDV2_ERR_OUT_OF_RANGE;
   for (int i = 0; i < p->rows; ++i) {
     if (p->start_frame[i] < 0 || p->start_frame[i] + p->grid_f > p->freq_rows) return SDV2_ERR_OUT_OF_RANGE;
-    if (p->dst_start[i] < 0 || p->dst_start[i] + p->tokens > p->cache_tokens) return SDV2_ERR_OUT_OF_RANGE;
+    if (with_kv && (p->dst_start[i] < 0 || p->dst_start[i] + p->tokens > p->cache_tokens))
+      return SDV2_ERR_OUT_OF_RANGE;
   }
 
   AppendKernelArgs a{};
@@ -281,7 +296,7 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
   a.split_h = a.split_t + third;
   for (int i = 0; i < p->rows; ++i) {
     a.start_frame[i] = p->start_frame[i];
-    a.dst_start[i] = p->dst_start[i];
+    a.dst_start[i] = with_kv ? p->dst_start[i] : 0;
     a.new_global[i] = p->new_global_end ? p->new_global_end[i] : 0;
     a.new_local[i] = p->new_local_end ? p->new_local_end[i] : 0;
   }
@@ -308,12 +323,17 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
     else launch(std::integral_constant<int, kNormMaxSteps>{});
     return hipGetLastError() == hipSuccess ? SDV2_OK : SDV2_ERR_LAUNCH;
   }
+  auto launch = [&](auto kernel) {
+    sdv2::launch_timed(kernel, grid, block, 0, stream, p->timing_start, p->timing_stop, a);
+  };
   if (p->dtype == SDV2_BF16) {
-    if (with_q) sdv2::launch_timed(kv_append_rope_kernel<uint16_t, true>, grid, block, 0, stream, p->timing_start, p->timing_stop, a);
-    else sdv2::launch_timed(kv_append_rope_kernel<uint16_t, false>, grid, block, 0, stream, p->timing_start, p->timing_stop, a);
+    if (!with_kv) launch(kv_append_rope_kernel<uint16_t, true, false>);
+    else if (with_q) launch(kv_append_rope_kernel<uint16_t, true, true>);
+    else launch(kv_append_rope_kernel<uint16_t, false, true>);
   } else {
-    if (with_q) sdv2::launch_timed(kv_append_rope_kernel<float, true>, grid, block, 0, stream, p->timing_start, p->timing_stop, a);
-    else sdv2::launch_timed(kv_append_rope_kernel<float, false>, grid, block, 0, stream, p->timing_start, p->timing_stop, a);
+    if (!with_kv) launch(kv_append_rope_kernel<float, true, false>);
+    else if (with_q) launch(kv_append_rope_kernel<float, true, true>);
+    else launch(kv_append_rope_kernel<float, false, true>);
   }
   return hipGetLastError() == hipSuccess ? SDV2_OK : SDV2_ERR_LAUNCH;
 }

@@ -197,6 +197,65 @@ def kv_append_rope(
     return q_out
 
 
+def causal_rope_apply(x: torch.Tensor, grid_sizes, freqs: torch.Tensor, start_frame=0, rope_cache=None) -> torch.Tensor:
+    """The reference's ``causal_rope_apply`` (causal_model.py:94-108) as one
+    launch per run of rows with the same grid: row i of ``x`` [B, L, H, 128]
+    is rotated over its first f*h*w tokens for ``grid_sizes[i]`` = (f, h, w)
+    starting at frame ``start_frame`` (an int, or one entry per row); later
+    tokens and rows without a grid are returned as they are.  Bit-identical to
+    the reference's complex128 product rounded to ``x``'s dtype.
+
+    ``freqs`` is the model's complex128 table or :func:`device_freqs` output.
+    ``rope_cache`` (the reference's pre-expanded per-token factors) is accepted
+    and not used: the kernel indexes the table itself.  The KV-cache path does
+    not call this: its append rotates q and k while it writes the cache.
+    """
+    dev = _require_gpu(x)
+    if x.dtype not in _DTYPES:
+        raise RuntimeError(f"unsupported dtype {x.dtype}")
+    rows, length, heads, _ = x.shape
+    grids = grid_sizes.tolist() if isinstance(grid_sizes, torch.Tensor) else [list(g) for g in grid_sizes]
+    grids = [tuple(int(n) for n in g) for g in grids][:rows]
+    if isinstance(start_frame, torch.Tensor):
+        starts = [int(s) for s in start_frame.reshape(-1).tolist()][:len(grids)]
+        grids = grids[:len(starts)]                    # the reference zips the two
+    else:
+        starts = [int(start_frame)] * len(grids)
+    for f, h, w in grids:
+        if min(f, h, w) <= 0 or f * h * w > length:
+            raise RuntimeError(f"grid {(f, h, w)} does not fit {length} tokens")
+    table = freqs if freqs.dtype == torch.float64 and freqs.device == dev else device_freqs(freqs, dev)
+    if table.dim() != 3 or tuple(table.shape[1:]) != (HEAD_DIM // 2, 2) or not table.is_contiguous():
+        raise RuntimeError("freqs must be the complex128 table or the float64 view from device_freqs()")
+    _stride3(x, "x")
+    whole = len(grids) == rows and all(f * h * w == length for f, h, w in grids)
+    out = torch.empty_like(x) if whole else x.clone()
+    if out.stride() != x.stride():
+        raise RuntimeError("x must be dense (its copy did not keep the strides)")
+
+    lib = _capi.lib()
+    with torch.cuda.device(dev):
+        r0 = 0
+        while r0 < len(grids):
+            r1 = r0 + 1
+            while r1 < len(grids) and r1 - r0 < _capi.MAX_ROWS and grids[r1] == grids[r0]:
+                r1 += 1
+            f, h, w = grids[r0]
+            p = _capi.AppendParams()
+            p.q_in, p.q_in_stride = x[r0:r1].data_ptr(), _stride3(x, "x")
+            p.q_out, p.q_out_stride = out[r0:r1].data_ptr(), _stride3(out, "out")
+            p.freqs, p.freq_rows = table.data_ptr(), table.shape[0]
+            p.dtype = _DTYPES[x.dtype]
+            p.rows, p.tokens, p.heads, p.head_dim = r1 - r0, f * h * w, heads, HEAD_DIM
+            p.grid_f, p.grid_h, p.grid_w = f, h, w
+            sf = _i64_array(starts[r0:r1])
+            p.start_frame = C.cast(sf, C.POINTER(C.c_int64))
+            p.stream = _stream_ptr(dev)
+            _capi.check(lib.sdv2_kv_append_rope(C.byref(p)), "sdv2_kv_append_rope")
+            r0 = r1
+    return out
+
+
 _WORKSPACES: dict = {}
 
 

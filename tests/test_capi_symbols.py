@@ -62,6 +62,20 @@ def test_argument_validation_without_gpu():
     assert lib.sdv2_kv_append_rope(C.byref(p)) == _capi.SDV2_ERR_INVALID_ARG
     p.rows, p.grid_f, p.grid_h, p.grid_w = 1, 1, 2, 3      # 6 != 8 tokens
     assert lib.sdv2_kv_append_rope(C.byref(p)) == _capi.SDV2_ERR_INVALID_ARG
+    # rotation of q alone: no k, v, caches - and then no index, norm or device slot either
+    r = _capi.AppendParams()
+    r.head_dim, r.rows, r.tokens, r.heads = 128, 1, 6, 1
+    r.grid_f, r.grid_h, r.grid_w = 1, 2, 3
+    r.freqs = 256
+    assert lib.sdv2_kv_append_rope(C.byref(r)) == _capi.SDV2_ERR_INVALID_ARG     # nothing to rotate
+    r.q_in, r.q_out = 256, 512
+    r.k_in = 768                                                                # k without v and the caches
+    assert lib.sdv2_kv_append_rope(C.byref(r)) == _capi.SDV2_ERR_INVALID_ARG
+    r.k_in = None
+    r.global_end_index = 1024
+    assert lib.sdv2_kv_append_rope(C.byref(r)) == _capi.SDV2_ERR_INVALID_ARG     # an index without a cache
+    r.global_end_index = None
+    assert lib.sdv2_kv_append_rope(C.byref(r)) == _capi.SDV2_ERR_INVALID_ARG     # no start_frame
     a = _capi.AttnParams()
     a.head_dim = 96
     assert lib.sdv2_swa_attn_fwd(C.byref(a)) == _capi.SDV2_ERR_UNSUPPORTED

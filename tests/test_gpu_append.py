@@ -203,3 +203,39 @@ def test_append_slot_chosen_on_the_device(gpu_device, fused_norm):
     with pytest.raises(RuntimeError):       # not on the device
         ops.kv_append_rope(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), kc, vc, table, grid, start_frames,
                            host_dst, dst_start_override=override)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_stand_alone_rotation_matches_oracle_bitwise(gpu_device, dtype):
+    """``causal_rope_apply`` on its own, called the way the reference calls it
+    (causal_model.py:253-259): rows with different grids, a tensor of start
+    frames, tokens past a row's grid and a row without a grid stay as they
+    are, and no cache is involved."""
+    from streamdiffusionv2_amd import ops
+
+    torch.manual_seed(31)
+    heads, length = 5, 150
+    grids = [(2, 5, 12), (2, 5, 12), (3, 5, 10), (1, 6, 8)]          # 120, 120, 150, 48 tokens
+    x = torch.randn(5, length, heads, 128).to(dtype)                 # the fifth row has no grid
+    starts = [3, 17, 0, 1000]
+    freqs = oracle.build_freqs()
+    want = oracle.causal_rope_apply(x, grids, freqs, starts)
+
+    got = ops.causal_rope_apply(x.to(gpu_device), torch.tensor(grids), freqs,
+                                start_frame=torch.tensor(starts, device=gpu_device), rope_cache=[("unused",)])
+    torch.cuda.synchronize()
+    assert got.dtype == dtype and got.shape == x.shape
+    assert torch.equal(_bits(got.cpu()), _bits(want))
+    assert torch.equal(_bits(got.cpu()[4]), _bits(x[4]))
+
+    # one start frame for all rows, the table already on the device, every row covered in full
+    y = torch.randn(3, 48, heads, 128).to(dtype)
+    want = oracle.causal_rope_apply(y, [(1, 6, 8)] * 3, freqs, [11] * 3)
+    got = ops.causal_rope_apply(y.to(gpu_device), [(1, 6, 8)] * 3, ops.device_freqs(freqs, gpu_device), start_frame=11)
+    torch.cuda.synchronize()
+    assert torch.equal(_bits(got.cpu()), _bits(want))
+
+    with pytest.raises(RuntimeError, match="does not fit"):
+        ops.causal_rope_apply(y.to(gpu_device), [(2, 6, 8)] * 3, freqs)
+    with pytest.raises(RuntimeError, match="status -3"):             # frame 1020 + 5 is past the 1024-row table
+        ops.causal_rope_apply(x.to(gpu_device), [(5, 5, 6)], freqs, start_frame=1020)
