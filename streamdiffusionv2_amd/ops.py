@@ -635,6 +635,11 @@ def flash_attn_with_kvcache(q, k_cache, v_cache, cache_seqlens=None):
     return swa_attention(q, k_cache, v_cache, cache_seqlens)
 
 
+# the reference's own fallback operator has the same four arguments and result
+# (causal_model.py:111-157); with this package both names are one kernel
+attention_with_kvcache_fallback = flash_attn_with_kvcache
+
+
 def flash_attention(q, k, v, q_lens=None, k_lens=None, dropout_p=0.0, softmax_scale=None, q_scale=None,
                     causal=False, window_size=(-1, -1), deterministic=False, dtype=torch.bfloat16, version=None):
     """The reference's generic attention entry (wan_base/modules/attention.py,

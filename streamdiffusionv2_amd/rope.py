@@ -24,6 +24,12 @@ def axis_table(positions: int, dim: int, theta: float = 10000.0) -> torch.Tensor
     return torch.polar(torch.ones_like(angle), angle)
 
 
+def rope_params(max_seq_len: int, dim: int, theta: float = 10000.0) -> torch.Tensor:
+    """The reference's name and argument order for :func:`axis_table`
+    (models/wan/wan_base/modules/model.py:29-36)."""
+    return axis_table(max_seq_len, dim, theta)
+
+
 def column_split(pairs: int) -> Tuple[int, int, int]:
     """How many of the ``pairs`` complex columns belong to (t, h, w)."""
     third = pairs // 3

@@ -118,3 +118,20 @@ def test_double_to_bf16_goes_through_float():
     bits = big.float().to(torch.bfloat16).view(torch.int16).tolist()
     for val, b in zip(big.tolist()[:256], bits[:256]):
         assert (b & 0xFFFF) == bf16_bits_from_f32(f32_round(val))
+
+
+def test_package_table_is_the_oracle_table_bit_for_bit():
+    """The package builds its table on the host with its own code; the GPU
+    parity tests hand either table to the kernels, so the two must be one."""
+    from streamdiffusionv2_amd import ops, rope
+
+    for head_dim, positions in ((128, 1024), (128, 64), (96, 33)):
+        mine = torch.view_as_real(rope.build_freqs(head_dim, positions))
+        theirs = torch.view_as_real(oracle.build_freqs(head_dim, positions))
+        assert torch.equal(mine.view(torch.int64), theirs.view(torch.int64))
+    assert rope.column_split(64) == (22, 21, 21)
+    # reference names (model.py:29-36, causal_model.py:111) resolve to the same code
+    assert torch.equal(torch.view_as_real(rope.rope_params(50, 44)), torch.view_as_real(oracle.rope_params(50, 44)))
+    with pytest.raises(ValueError):
+        rope.rope_params(8, 7)
+    assert ops.attention_with_kvcache_fallback is ops.flash_attn_with_kvcache
