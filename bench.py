@@ -511,6 +511,9 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU (the KV-cache path has no CPU fallback)", file=sys.stderr)
         sys.exit(2)
+    from streamdiffusionv2_amd import build_ext
+
+    build_ext.ensure_built()       # the library normally comes with the tree; compile only when it is absent
     if args.calibrate_copy:
         from streamdiffusionv2_amd import ops
 

@@ -58,6 +58,14 @@ def build(verbose: bool = False, keep_temps: bool = False) -> Path:
     return LIB_PATH
 
 
+def ensure_built(verbose: bool = False) -> Path:
+    """Build the library only when none is there.  For the entry points around
+    the package (smoke run, benchmark, GPU test session): the package itself
+    never builds behind the caller's back, it raises when the library is
+    missing."""
+    return LIB_PATH if LIB_PATH.exists() else build(verbose)
+
+
 GPU_CALLER_SRC = REPO_ROOT / "tests" / "c_abi" / "gpu_caller.cpp"
 GPU_CALLER_BIN = REPO_ROOT / "tests" / "c_abi" / "_bin" / "gpu_caller"
 

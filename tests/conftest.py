@@ -18,7 +18,8 @@ def gpu_device():
 
     if not torch.cuda.is_available():
         pytest.skip("no GPU visible")
-    from streamdiffusionv2_amd import _capi
+    from streamdiffusionv2_amd import _capi, build_ext
 
-    _capi.lib()  # fail loudly when the HIP extension is missing
+    build_ext.ensure_built()   # a GPU box normally gets the library with the tree; build only when it did not
+    _capi.lib()                # fail loudly when the HIP extension is missing
     return torch.device("cuda:0")

@@ -188,3 +188,16 @@ def test_documented_ctypes_struct_matches_the_binding():
     block = block[:block.index("p = AttnParams(")]
     documented = re.findall(r'\("(\w+)",', block)
     assert documented == [name for name, _ in _capi.AttnParams._fields_]
+
+
+def test_entry_points_build_only_when_no_library_is_there(monkeypatch, tmp_path):
+    """smoke(), bench.py and the GPU test session call ``ensure_built``: a
+    present library is loaded as it is, a missing one is compiled; the package
+    loader itself never compiles (it raises, see above)."""
+    from streamdiffusionv2_amd import build_ext
+
+    calls = []
+    monkeypatch.setattr(build_ext, "build", lambda verbose=False: calls.append(verbose) or build_ext.LIB_PATH)
+    assert build_ext.ensure_built() == build_ext.LIB_PATH and calls == []
+    monkeypatch.setattr(build_ext, "LIB_PATH", tmp_path / "libsdv2kv.so")
+    assert build_ext.ensure_built() == tmp_path / "libsdv2kv.so" and calls == [False]
