@@ -118,6 +118,10 @@ def test_cpu_tensors_are_refused():
     assert "DeviceType::CUDA" not in str(err.value)
     with pytest.raises(RuntimeError, match="GPU only"):
         ops.swa_attention(q, q, q)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ops.causal_rope_apply(q, [(1, 2, 4)], torch.zeros(4, 64, dtype=torch.complex128))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ops.attention_with_kvcache_fallback(q, q, q, None)
 
 
 def test_module_signature_matches_reference():
