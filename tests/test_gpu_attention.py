@@ -131,3 +131,59 @@ def test_attention_random_shapes(gpu_device):
         got = ops.swa_attention(q.to(gpu_device), kd, vd, sl, num_splits=splits, **kw)
         torch.cuda.synchronize()
         _check(got.cpu(), want)
+
+
+@pytest.mark.parametrize("name", ["c2_wan1.3b_1560tok_6frames", "c4_wan14b_1560tok_6frames"])
+def test_full_size_properties(gpu_device, name):
+    """At the benchmark's own sizes the CPU oracle is too slow for every row,
+    so the attention is checked through what the mathematics fixes at any
+    size: (i) a value that is the same for every key comes back unchanged,
+    whatever the scores; (ii) the result does not depend on the order of the
+    cache slots (a ring holds them in rotated order); (iii) it does not depend
+    on how many key ranges the call is split into; (iv) keys at and beyond a
+    row's length have no influence, whatever they hold."""
+    from streamdiffusionv2_amd import ops, workloads
+
+    w = next(x for x in workloads.WORKLOADS.values() if x.name == name)
+    rows, S, H, L = w.rows, w.chunk_tokens, w.heads, w.cache_tokens
+    gen = torch.Generator(device=gpu_device).manual_seed(77)
+
+    def rnd(*shape):
+        return (torch.randn(*shape, device=gpu_device, generator=gen) * 0.6).bfloat16()
+
+    q = rnd(rows, S, H, 128)
+    k = rnd(rows, H, L, 128).permute(0, 2, 1, 3)          # head-major, as the caches are
+    v = rnd(rows, H, L, 128).permute(0, 2, 1, 3)
+    base = ops.swa_attention(q, k, v, None).float()
+    assert torch.isfinite(base).all()
+
+    # (i) constant value per (row, head)
+    const = rnd(rows, H, 1, 128).expand(rows, H, L, 128).contiguous().permute(0, 2, 1, 3)
+    got = ops.swa_attention(q, k, const, None).float()
+    want = const[:, :1].float().expand(rows, S, H, 128)
+    assert (got - want).abs().max().item() <= MAX_ABS
+
+    # (ii) slots in another order: frames rotated by two, as a ring that has wrapped holds them
+    frame = w.grid[1] * w.grid[2]
+    order = torch.arange(L, device=gpu_device).roll(2 * frame)
+    kp = k[:, order].permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    vp = v[:, order].permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    rolled = ops.swa_attention(q, kp, vp, None).float()
+    err = (rolled - base).abs()
+    assert err.max().item() <= MAX_ABS and err.mean().item() <= MEAN_ABS
+
+    # (iii) one key range against the library's choice and a larger count
+    for splits in (1, 5):
+        other = ops.swa_attention(q, k, v, None, num_splits=splits).float()
+        err = (other - base).abs()
+        assert err.max().item() <= MAX_ABS and err.mean().item() <= MEAN_ABS, splits
+
+    # (iv) a row that is still filling: what lies beyond its length is never read into the result
+    lens = torch.full((rows,), L - frame - 7, dtype=torch.int32, device=gpu_device)
+    short = ops.swa_attention(q, k, v, lens).float()
+    k2, v2 = k.clone(), v.clone()
+    k2[:, L - frame - 7:] = 3.0e4                         # would dominate every softmax if it were seen
+    v2[:, L - frame - 7:] = float("nan")
+    again = ops.swa_attention(q, k2, v2, lens).float()
+    torch.cuda.synchronize()
+    assert torch.equal(short, again)
