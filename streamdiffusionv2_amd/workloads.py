@@ -78,6 +78,36 @@ def make_qkv(w: Workload, chunk: int, layer: int, seed: int = 0, rows: int = Non
     return q.to(w.dtype), k.to(w.dtype), v.to(w.dtype)
 
 
+class InputPool:
+    """Inputs for long streams without a random-number pass per call: one
+    seeded N(0,1) pool in the workload's dtype, of which q, k and v of every
+    (chunk, layer) are windows at distinct offsets (so no two calls see the same
+    tensors, and the GPU path and the CPU oracle see the same numbers).  The
+    outlier rows of a workload are drawn per call from its own seed."""
+
+    def __init__(self, w: Workload, seed: int = 0, offsets: int = 1 << 16):
+        self.w = w
+        self.n = w.rows * w.chunk_tokens * w.heads * 128
+        self.span = 8 * offsets
+        gen = torch.Generator().manual_seed(seed)
+        self.pool = (torch.randn(3 * (self.n + self.span), generator=gen) * w.input_scale).to(w.dtype)
+        self.seed = seed
+
+    def qkv(self, chunk: int, layer: int, rows: int = None):
+        w = self.w
+        rows = w.rows if rows is None else rows
+        n = rows * w.chunk_tokens * w.heads * 128
+        off = 8 * ((chunk * 7919 + layer * 104729 + 13) % (self.span // 8))
+        shape = (rows, w.chunk_tokens, w.heads, 128)
+        q, k, v = (self.pool[off + j * (self.n + self.span):][:n].view(shape) for j in range(3))
+        if w.outlier_fraction > 0:
+            gen = torch.Generator().manual_seed(self.seed + 1000 * chunk + layer)
+            hot = torch.rand((rows, w.chunk_tokens), generator=gen) < w.outlier_fraction
+            k = k.clone()
+            k[hot] = k[hot] * 8.0
+        return q, k, v
+
+
 def row_chunks(w: Workload, call: int) -> List[int]:
     """Chunk number each row works on at call ``call`` of a staggered stream
     batch.  Call 0 is the first chunk on every row (the reference runs it once

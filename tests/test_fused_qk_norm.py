@@ -56,7 +56,7 @@ def _ulp_diff_bf16(a, b):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("heads", [12, 40, 5])
+@pytest.mark.parametrize("heads", [12, 40, 5, 48, 64])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_fused_norm_append(gpu_device, heads, dtype):
     from streamdiffusionv2_amd import ops, ring, rope

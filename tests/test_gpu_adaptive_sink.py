@@ -22,13 +22,13 @@ THR = 0.2
 MARGIN = 0.03
 
 
-def directed_chunk(gen, rows, heads, dtype, basis, scene=None, scale=0.25):
-    """q, k, v [rows, FT, heads, 128]: noise plus a chunk-wide direction from
+def directed_chunk(gen, rows, heads, dtype, basis, scene=None, scale=0.25, ft=FT):
+    """q, k, v [rows, ft, heads, 128]: noise plus a chunk-wide direction from
     the span of `basis` (the same on every token, so it survives the frame
     mean; RoPE averages part of k's away).  With `scene` (coefficients [3]) the
     direction stays near that scene's, so consecutive chunks look alike until
     the scene changes."""
-    shape = (rows, FT, heads, 128)
+    shape = (rows, ft, heads, 128)
     q = torch.randn(shape, generator=gen) * scale
     k = torch.randn(shape, generator=gen) * scale
     v = torch.randn(shape, generator=gen) * scale
@@ -65,22 +65,23 @@ def test_stream_recipe_has_clear_margins_on_the_oracle():
         assert 0 < refreshed < len(sims)
 
 
-def _oracle_stream(dtype, seed, rows, calls, heads=2, sink=3, cache_frames=6):
+def _oracle_stream(dtype, seed, rows, calls, heads=2, sink=3, cache_frames=6, grid=GRID, with_attention=True):
+    ft = grid[1] * grid[2]
     gen = torch.Generator().manual_seed(seed)
     basis = torch.randn(3, heads * 128, generator=gen)
     freqs = oracle.build_freqs()
-    cache = oracle.new_kv_cache(1, 1, cache_frames * FT, heads, 1, dtype=dtype)[0]
+    cache = oracle.new_kv_cache(1, 1, cache_frames * ft, heads, 1, dtype=dtype)[0]
     layer = oracle.RingAttentionOracle(sink_size=sink, adapt_sink_thr=THR)
     record, sims, refreshed = [], [], 0
     for call in range(calls):
         if call == 1 and rows > 1:
             oracle.replicate_for_stream_batch([cache], rows)
         n = 1 if call == 0 else rows
-        starts = [max(call - r, 0) * FT for r in range(n)]
+        starts = [max(call - r, 0) * ft for r in range(n)]
         if call % 4 == 0:
             scene = torch.randn(3, generator=gen)       # a scene cut every fourth chunk
-        q, k, v = directed_chunk(gen, n, heads, dtype, basis, scene)
-        out, roped_q, seq = layer.step(q, k, v, [GRID] * n, freqs, cache, starts)
+        q, k, v = directed_chunk(gen, n, heads, dtype, basis, scene, ft=ft)
+        out, roped_q, seq = layer.step(q, k, v, [grid] * n, freqs, cache, starts, with_attention=with_attention)
         sims.extend(layer.last_sims)
         refreshed += sum(1 for s in layer.last_sims if s.min().item() < THR)
         record.append(dict(q=q, k=k, v=v, starts=starts, out=out, roped_q=roped_q, seq=seq,
@@ -252,4 +253,121 @@ def test_stream_with_refresh(gpu_device, seed, rows, look_every_call):
         want = oracle.attention_fp32_reference(rec["roped_q"], rec["cache_k"], rec["cache_v"], rec["seq"])
         unit = max(1.0, want.abs().max().item())
         err = (got.float().cpu() - want).abs()
+        assert err.max().item() <= 2e-2 * unit and err.mean().item() <= 2e-3 * unit, call
+
+
+# --------------------------------------------------------------------------
+# The shipped shape: 480p latent frames of 30 x 52 = 1560 tokens, sink 3,
+# threshold 0.2 (configs/wan_causal_dmd_v2v.yaml:53-56), 12 heads (Wan 1.3B)
+# and 40 heads (Wan 14B).  At this frame size every workgroup of the frame-sum
+# kernel runs its four-tokens-in-flight main loop (195 tokens per workgroup)
+# and 40 heads take the wide build of the decision kernel.
+# --------------------------------------------------------------------------
+PROD_GRID = (1, 30, 52)
+PROD_FT = 1560
+PROD_STREAMS = [(12, 23, 12), (40, 23, 10)]          # heads, seed, calls
+
+
+def test_production_stream_recipe_has_clear_margins_on_the_oracle():
+    for heads, seed, calls in PROD_STREAMS:
+        sims, refreshed = _oracle_stream(torch.bfloat16, seed, 1, calls, heads=heads, grid=PROD_GRID,
+                                         with_attention=False)[1:]
+        assert oracle_margins_ok(sims), [s.tolist() for s in sims]
+        assert 0 < refreshed < len(sims)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("heads", [12, 40])
+@pytest.mark.parametrize("head_major", [True, False])
+def test_similarity_operator_production_shape(gpu_device, heads, head_major):
+    from streamdiffusionv2_amd import ops, rope
+
+    print(f"sink similarity operator at 1560-token frames: heads={heads} head_major={head_major}", flush=True)
+    rows, sink, frames = 2, 3, 6
+    gen = torch.Generator().manual_seed(300 + heads)
+    basis = torch.randn(3, heads * 128, generator=gen)
+    _, k, v = directed_chunk(gen, rows, heads, torch.bfloat16, basis, ft=PROD_FT)
+    ck = torch.cat([directed_chunk(gen, rows, heads, torch.bfloat16, basis, ft=PROD_FT)[1] for _ in range(frames)], dim=1)
+    cv = torch.cat([directed_chunk(gen, rows, heads, torch.bfloat16, basis, ft=PROD_FT)[2] for _ in range(frames)], dim=1)
+    start_frames = [17, 3]
+    roped = oracle.causal_rope_apply(k, [PROD_GRID] * rows, oracle.build_freqs(), start_frames).type_as(v)
+    want = []
+    for r in range(rows):
+        def means(t, n):
+            return t.reshape(n, PROD_FT, -1).mean(1)
+        sk = torch.cosine_similarity(means(ck[r:r + 1, :sink * PROD_FT], sink), means(roped[r:r + 1], 1), dim=-1)
+        sv = torch.cosine_similarity(means(cv[r:r + 1, :sink * PROD_FT], sink), means(v[r:r + 1], 1), dim=-1)
+        want.append(((sk + sv) / 2).float())
+    want = torch.stack(want)
+
+    def on_gpu(t):
+        if head_major:
+            return t.permute(0, 2, 1, 3).contiguous().to(gpu_device).permute(0, 2, 1, 3)
+        return t.to(gpu_device)
+
+    table = ops.device_freqs(rope.build_freqs(), gpu_device)
+    override = torch.full((rows,), 777, dtype=torch.int64, device=gpu_device)
+    sim, refresh = ops.sink_similarity(k.to(gpu_device), v.to(gpu_device), on_gpu(ck), on_gpu(cv), table,
+                                       PROD_GRID[1:], start_frames, sink, 1.5, dst_start_override=override,
+                                       override_rows=[True, True])
+    torch.cuda.synchronize()
+    assert (sim.cpu() - want).abs().max().item() <= 1e-2, (sim.cpu(), want)
+    got = refresh.cpu().tolist()
+    assert got == sim.argmin(dim=1).cpu().tolist()            # threshold 1.5: always the minimum
+    assert override.cpu().tolist() == [g * PROD_FT for g in got]
+    for r in range(rows):
+        s = want[r].sort().values
+        if (s[1] - s[0]).item() > MARGIN:
+            assert got[r] == int(want[r].argmin())
+    # the shipped threshold
+    _, shipped = ops.sink_similarity(k.to(gpu_device), v.to(gpu_device), on_gpu(ck), on_gpu(cv), table,
+                                     PROD_GRID[1:], start_frames, sink, THR)
+    for r in range(rows):
+        lo = want[r].min().item()
+        s = want[r].sort().values
+        if abs(lo - THR) > MARGIN and (lo >= THR or (s[1] - s[0]).item() > MARGIN):
+            assert shipped[r].item() == (int(want[r].argmin()) if lo < THR else -1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("heads,seed,calls", PROD_STREAMS)
+def test_stream_with_refresh_production_shape(gpu_device, heads, seed, calls):
+    """The shipped configuration as a stream: 1560-token frames, cache of six
+    frames of which three are sink frames, threshold 0.2.  The ring fills
+    (calls 0-5) and then evicts; scene cuts every fourth chunk make the check
+    refresh a sink frame on some calls and keep all three on others.  Decision,
+    queue, slot, indices and the cache bits are compared after every call; the
+    attention on a seeded sample of query rows."""
+    from streamdiffusionv2_amd import ring, rope
+    from streamdiffusionv2_amd.attention import RingKVPath
+
+    print(f"adaptive sink stream at 1560-token frames: heads={heads} calls={calls}", flush=True)
+    sink, cache_frames = 3, 6
+    record, sims, refreshed = _oracle_stream(torch.bfloat16, seed, 1, calls, heads=heads, grid=PROD_GRID,
+                                             with_attention=False)
+    assert oracle_margins_ok(sims) and 0 < refreshed < len(sims)
+    assert any(a < sink * PROD_FT for rec in record[cache_frames:] for a, _ in rec["writes"])   # a sink frame is rewritten
+
+    freqs = rope.build_freqs()
+    cache = ring.new_kv_cache(1, 1, cache_frames * PROD_FT, heads, 1, device=gpu_device)[0]
+    path = RingKVPath(sink_size=sink, adapt_sink_thr=THR)
+    gen = torch.Generator().manual_seed(5)
+    for call, rec in enumerate(record):
+        got, got_q = path.attend(rec["q"].to(gpu_device), rec["k"].to(gpu_device), rec["v"].to(gpu_device),
+                                 torch.tensor([PROD_GRID]), freqs, cache, rec["starts"], return_roped_query=True)
+        torch.cuda.synchronize()
+        want_refresh = [int(s.argmin()) if s.min().item() < THR else -1 for s in rec["sims"]]
+        if call % 2 == 0 or call == len(record) - 1:          # every other call settles lazily, as in a running stream
+            assert path.last_refresh == want_refresh, call
+            assert path.evict_idx == rec["queue"], call
+            assert [(a, a + PROD_FT) for a in path.last_plan.dst_start] == rec["writes"], call
+        assert cache["global_end_index"].tolist() == [rec["starts"][0] + PROD_FT], call
+        assert cache["local_end_index"].tolist() == rec["seq"], call
+        assert torch.equal(got_q.cpu().view(torch.int16), rec["roped_q"].view(torch.int16)), call
+        for name in ("k", "v"):
+            assert torch.equal(cache[name].cpu().view(torch.int16), rec["cache_" + name].view(torch.int16)), (call, name)
+        idx = torch.randperm(PROD_FT, generator=gen)[:32].sort().values
+        want = oracle.attention_fp32_reference(rec["roped_q"][:, idx], rec["cache_k"], rec["cache_v"], rec["seq"])
+        unit = max(1.0, want.abs().max().item())
+        err = (got[:, idx.to(gpu_device)].float().cpu() - want).abs()
         assert err.max().item() <= 2e-2 * unit and err.mean().item() <= 2e-3 * unit, call

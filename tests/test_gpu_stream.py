@@ -25,11 +25,17 @@ def _bits(t):
     return t.contiguous().view(torch.int16 if t.dtype == torch.bfloat16 else torch.int32)
 
 
-def _run(w, gpu_device, layers, calls, sample_rows=None, full_compare_at=None):
+def _run(w, gpu_device, layers, calls, sample_rows=None, full_compare_at=None, pool=None, first_layer=0,
+         attention_every=1):
+    """`pool` (workloads.InputPool) replaces the per-call random draw for long
+    streams; `first_layer` offsets the layer number that selects the inputs;
+    with `attention_every` = n the attention output is checked on every n-th
+    call and on the last one (the cache state is checked on every call)."""
     from streamdiffusionv2_amd import ring, rope
     from streamdiffusionv2_amd.attention import RingKVPath
 
-    print(f"stream parity: {w.name} layers={layers} calls={calls} sample={sample_rows}", flush=True)
+    print(f"stream parity: {w.name} layers={first_layer}..{first_layer + layers - 1} calls={calls} "
+          f"sample={sample_rows}", flush=True)
     freqs = rope.build_freqs()
     B, S = w.rows, w.chunk_tokens
     g_caches = ring.new_kv_cache(layers, 1, w.cache_tokens, w.heads, 1, dtype=w.dtype, device=gpu_device)
@@ -46,7 +52,10 @@ def _run(w, gpu_device, layers, calls, sample_rows=None, full_compare_at=None):
         rows = 1 if (call == 0 and B > 1) else B
         starts = workloads.row_starts(w, call)[:rows]
         for layer in range(layers):
-            q, k, v = workloads.make_qkv(w, call, layer, rows=rows)
+            if pool is None:
+                q, k, v = workloads.make_qkv(w, call, first_layer + layer, rows=rows)
+            else:
+                q, k, v = pool.qkv(call, first_layer + layer, rows=rows)
             got, got_q = g_paths[layer].attend(
                 q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), torch.tensor(grids[:rows]), freqs,
                 g_caches[layer], starts, return_roped_query=True)
@@ -68,6 +77,8 @@ def _run(w, gpu_device, layers, calls, sample_rows=None, full_compare_at=None):
                 for name in ("k", "v"):
                     assert torch.equal(g_caches[layer][name], o_caches[layer][name].to(gpu_device)), (call, name)
             # attention
+            if call % attention_every and call != calls - 1:
+                continue
             if sample_rows is None:
                 idx = torch.arange(S)
             else:
@@ -122,6 +133,33 @@ def test_c3_full_size(gpu_device):
 def test_c5_full_size_with_outliers(gpu_device):
     w = workloads.WORKLOADS[5]
     _run(w, gpu_device, layers=1, calls=9, sample_rows=24, full_compare_at={0, 7, 8})
+
+
+def _wrap_calls(w, calls):
+    """Calls at which the ring starts a new round over its rotating slots."""
+    slots = w.cache_tokens // w.chunk_tokens
+    return {c for c in range(slots, calls + w.rows) if (c - slots) % (slots - 1) == 0}
+
+
+@pytest.mark.parametrize("first_layer", [0, 10, 20])
+def test_c2_stated_length(gpu_device, first_layer):
+    """Config 2 as stated: 30 layers (ten per case) x 50 chunks, so the ring
+    of five rotating slots goes round nine times.  Cache compared in full at the
+    first call, at every wrap and at the end."""
+    w = workloads.WORKLOADS[2]
+    assert w.layers == 30 and w.chunks == 50
+    _run(w, gpu_device, layers=10, calls=w.chunks, sample_rows=8, first_layer=first_layer,
+         full_compare_at={0, w.chunks - 1} | _wrap_calls(w, w.chunks), pool=workloads.InputPool(w, seed=first_layer))
+
+
+@pytest.mark.parametrize("cfg,first_layer", [(4, 0), (4, 1), (3, 0), (3, 1), (5, 0), (5, 1)])
+def test_c3_c4_c5_stated_chunk_counts(gpu_device, cfg, first_layer):
+    """Configs 3, 4 and 5 over their stated 40 / 30 / 25 chunks, two layers
+    each (one per case)."""
+    w = workloads.WORKLOADS[cfg]
+    _run(w, gpu_device, layers=1, calls=w.chunks, sample_rows=16 if cfg == 4 else 8, first_layer=first_layer,
+         full_compare_at={0, w.chunks - 1} | _wrap_calls(w, w.chunks), pool=workloads.InputPool(w, seed=cfg),
+         attention_every=1 if cfg == 4 else 5)
 
 
 def test_kernel_timers_measure_each_kernel(gpu_device):
