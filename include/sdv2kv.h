@@ -3,8 +3,8 @@
  * causal Wan DiT of StreamDiffusionV2.
  *
  * Four operators, all enqueued on a caller-supplied HIP stream, all working
- * on caller-owned device memory (the library owns nothing and keeps no
- * mutable state):
+ * on caller-owned device memory (the library keeps no state between calls; the
+ * one entry point that brings its own scratch memory says so):
  *
  *   sdv2_kv_append_rope   fused RoPE-on-write chunk append
  *   sdv2_swa_attn_fwd     chunk-Q x (sink + window) K/V flash attention
@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SDV2KV_ABI_VERSION 5
+#define SDV2KV_ABI_VERSION 6
 #define SDV2_HEAD_DIM 128      /* causal_stream_inference.py:99-100 fixes 128 */
 #define SDV2_MAX_ROWS 16       /* rows (B) per sdv2_kv_append_rope call       */
 #define SDV2_MAX_SINK_FRAMES 16 /* sink frames per sdv2_sink_similarity call  */
@@ -43,7 +43,9 @@ typedef enum sdv2_status {
   SDV2_ERR_OUT_OF_RANGE = -3,  /* write range outside the cache, RoPE row     */
                                /* beyond the table                            */
   SDV2_ERR_WORKSPACE = -4,     /* split-KV workspace missing or too small     */
-  SDV2_ERR_LAUNCH = -5         /* hipLaunchKernel reported an error           */
+  SDV2_ERR_LAUNCH = -5,        /* hipLaunchKernel reported an error           */
+  SDV2_ERR_SCRATCH_LIMIT = -6  /* sdv2_swa_attn_fwd_static: the call needs    */
+                               /* more than SDV2_STATIC_SCRATCH_BYTES         */
 } sdv2_status;
 
 typedef enum sdv2_dtype {
@@ -195,6 +197,26 @@ int sdv2_swa_attn_default_splits(int32_t rows, int32_t q_tokens, int32_t heads, 
 size_t sdv2_swa_attn_workspace_bytes(int32_t rows, int32_t q_tokens, int32_t heads,
                                      int32_t max_seq_len, int32_t num_splits);
 int sdv2_swa_attn_fwd(const sdv2_attn_params* p);
+
+/* ------------------------------------------------------------------------
+ * sdv2_swa_attn_fwd for callers that cannot allocate.  No counterpart in the
+ * reference: it is for code under HIP graph capture, tight serving loops and
+ * harnesses that forbid hipMalloc, which cannot size and bring the workspace
+ * a split call needs.  Same arguments, kernels and results as
+ * sdv2_swa_attn_fwd, except that `workspace` / `workspace_bytes` are ignored:
+ * the partial results of a split call go to SDV2_STATIC_SCRATCH_BYTES of
+ * device memory that the library itself holds on every GPU it runs on, from
+ * load to process exit.  A call whose sdv2_swa_attn_workspace_bytes() exceeds
+ * that returns SDV2_ERR_SCRATCH_LIMIT and launches nothing (64 MiB covers the
+ * Wan 1.3B and 14B shapes at 480p: one row of a 1560-token chunk against six
+ * frames).  The call allocates and frees nothing and does not synchronise.
+ * Nothing in the scratch has to be cleared between calls (the merge reads only
+ * what the same call's attention kernel wrote), but all calls on one GPU share
+ * it: two calls that overlap in time on one GPU - different streams, threads
+ * or processes' graphs replayed concurrently - race.
+ * ---------------------------------------------------------------------- */
+#define SDV2_STATIC_SCRATCH_BYTES (64u << 20)
+int sdv2_swa_attn_fwd_static(const sdv2_attn_params* p);
 
 /* ------------------------------------------------------------------------
  * Adaptive sink refresh decision.

@@ -11,7 +11,7 @@ from typing import Optional
 
 LIB_PATH = Path(__file__).resolve().parent / "_lib" / "libsdv2kv.so"
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 HEAD_DIM = 128
 MAX_ROWS = 16
 
@@ -21,6 +21,8 @@ SDV2_ERR_UNSUPPORTED = -2
 SDV2_ERR_OUT_OF_RANGE = -3
 SDV2_ERR_WORKSPACE = -4
 SDV2_ERR_LAUNCH = -5
+SDV2_ERR_SCRATCH_LIMIT = -6
+STATIC_SCRATCH_BYTES = 64 << 20
 
 STAGE_ALL, STAGE_PARTIAL, STAGE_MERGE = 0, 1, 2
 
@@ -35,6 +37,7 @@ EXPORTED_SYMBOLS = (
     "sdv2_swa_attn_default_splits",
     "sdv2_swa_attn_workspace_bytes",
     "sdv2_swa_attn_fwd",
+    "sdv2_swa_attn_fwd_static",
     "sdv2_sink_similarity_workspace_bytes",
     "sdv2_sink_similarity",
     "sdv2_cache_relayout",
@@ -170,6 +173,8 @@ def lib() -> C.CDLL:
     handle.sdv2_swa_attn_workspace_bytes.argtypes = [C.c_int32] * 5
     handle.sdv2_swa_attn_fwd.restype = C.c_int
     handle.sdv2_swa_attn_fwd.argtypes = [C.POINTER(AttnParams)]
+    handle.sdv2_swa_attn_fwd_static.restype = C.c_int
+    handle.sdv2_swa_attn_fwd_static.argtypes = [C.POINTER(AttnParams)]
     handle.sdv2_sink_similarity_workspace_bytes.restype = C.c_size_t
     handle.sdv2_sink_similarity_workspace_bytes.argtypes = [C.c_int32] * 3
     handle.sdv2_sink_similarity.restype = C.c_int

@@ -24,6 +24,7 @@ extern "C" const char* sdv2_status_string(int status) {
     case SDV2_ERR_OUT_OF_RANGE: return "write range outside the cache or RoPE position beyond the table";
     case SDV2_ERR_WORKSPACE: return "split-KV workspace missing or too small";
     case SDV2_ERR_LAUNCH: return "kernel launch failed";
+    case SDV2_ERR_SCRATCH_LIMIT: return "the call needs more split-KV scratch than the library's static buffer holds";
     default: return "unknown status";
   }
 }

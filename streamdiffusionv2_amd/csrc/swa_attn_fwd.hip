@@ -43,6 +43,7 @@
 #include <stdint.h>
 
 #include <atomic>
+#include <mutex>
 #include <utility>
 
 #include "sdv2kv.h"
@@ -916,6 +917,38 @@ size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
 }  // namespace
 
+// Device memory the library owns, for sdv2_swa_attn_fwd_static: the partial
+// results of a split call when the caller cannot bring a workspace.  One copy
+// per GPU, at an address of its own on each, held until the process ends.  In
+// host code `scratch` is only a handle for hipGetSymbolAddress; kernels get the
+// address that call returns.
+static __device__ __align__(256) unsigned char scratch[SDV2_STATIC_SCRATCH_BYTES];
+
+namespace {
+
+// Address of `scratch` on the current device, looked up once per device with
+// that device current; nullptr when the runtime refuses.
+void* static_scratch_address() {
+  static std::mutex lock;
+  static void* address[kMaxDevices];
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> guard(lock);
+  if (!address[device]) {
+    void* ptr = nullptr;
+    if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    address[device] = ptr;
+  }
+  return address[device];
+}
+
+int attn_fwd(const sdv2_attn_params* p, void* workspace, size_t workspace_bytes);
+
+}  // namespace
+
 extern "C" int sdv2_swa_attn_default_splits(int32_t rows, int32_t q_tokens, int32_t heads, int32_t max_seq_len) {
   if (rows <= 0 || q_tokens <= 0 || heads <= 0 || max_seq_len <= 0) return 1;
   // One workgroup per CU.  With s key-range splits there are qwork * s
@@ -950,6 +983,27 @@ extern "C" size_t sdv2_swa_attn_workspace_bytes(int32_t rows, int32_t q_tokens, 
 
 extern "C" int sdv2_swa_attn_fwd(const sdv2_attn_params* p) {
   if (!p) return SDV2_ERR_INVALID_ARG;
+  return attn_fwd(p, p->workspace, p->workspace_bytes);
+}
+
+extern "C" int sdv2_swa_attn_fwd_static(const sdv2_attn_params* p) {
+  if (!p) return SDV2_ERR_INVALID_ARG;
+  if (p->rows <= 0 || p->q_tokens <= 0 || p->heads <= 0 || p->max_seq_len < 0)
+    return attn_fwd(p, nullptr, 0);                       // nothing to split: same answers as the plain entry point
+  const int splits = p->num_splits > 0 ? p->num_splits
+                                       : sdv2_swa_attn_default_splits(p->rows, p->q_tokens, p->heads, p->max_seq_len);
+  if (splits <= 1) return attn_fwd(p, nullptr, 0);
+  if (sdv2_swa_attn_workspace_bytes(p->rows, p->q_tokens, p->heads, p->max_seq_len, splits) >
+      (size_t)SDV2_STATIC_SCRATCH_BYTES)
+    return SDV2_ERR_SCRATCH_LIMIT;
+  void* ptr = static_scratch_address();
+  if (!ptr) return SDV2_ERR_LAUNCH;
+  return attn_fwd(p, ptr, SDV2_STATIC_SCRATCH_BYTES);
+}
+
+namespace {
+
+int attn_fwd(const sdv2_attn_params* p, void* workspace, size_t workspace_bytes) {
   if (p->head_dim != kD) return SDV2_ERR_UNSUPPORTED;
   if (p->rows < 0 || p->q_tokens < 0 || p->heads <= 0 || p->max_seq_len < 0) return SDV2_ERR_INVALID_ARG;
   if (p->rows == 0 || p->q_tokens == 0) return SDV2_OK;
@@ -991,10 +1045,10 @@ extern "C" int sdv2_swa_attn_fwd(const sdv2_attn_params* p) {
 
   if (splits > 1) {
     const size_t need = sdv2_swa_attn_workspace_bytes(p->rows, p->q_tokens, p->heads, p->max_seq_len, splits);
-    if (!p->workspace || p->workspace_bytes < need) return SDV2_ERR_WORKSPACE;
-    if (reinterpret_cast<uintptr_t>(p->workspace) & 255) return SDV2_ERR_INVALID_ARG;
+    if (!workspace || workspace_bytes < need) return SDV2_ERR_WORKSPACE;
+    if (reinterpret_cast<uintptr_t>(workspace) & 255) return SDV2_ERR_INVALID_ARG;
     const size_t nq = (size_t)p->rows * p->heads * p->q_tokens;
-    char* ws = static_cast<char*>(p->workspace);
+    char* ws = static_cast<char*>(workspace);
     a.part_o = reinterpret_cast<uint16_t*>(ws);
     ws += align_up((size_t)splits * nq * kD * sizeof(uint16_t), 256);
     a.part_lse = reinterpret_cast<float*>(ws);
@@ -1037,3 +1091,5 @@ extern "C" int sdv2_swa_attn_fwd(const sdv2_attn_params* p) {
   }
   return SDV2_OK;
 }
+
+}  // namespace

@@ -296,8 +296,15 @@ def swa_attention(
     stages: int = _capi.STAGE_ALL,
     chunk_key_start: Optional[torch.Tensor] = None,
     mask_block_tokens: int = 0,
+    static_scratch: bool = False,
 ) -> torch.Tensor:
     """out[b] = softmax(q[b] k_cache[b,:seq_lens[b]]^T * scale) v_cache[b,:seq_lens[b]].
+
+    ``static_scratch`` takes the library's allocation-free entry point
+    (``sdv2_swa_attn_fwd_static``): partial results of a split call go to device
+    memory the library holds itself (64 MiB per GPU, shared by all calls on
+    that GPU), no workspace is sized or allocated here; with ``out`` given the
+    whole call then allocates nothing.
 
     q [B,S,H,128] bf16; k_cache/v_cache [B,L,H,128] bf16 views with any row /
     token / head strides; seq_lens int32 [B] on the device (None = L).
@@ -323,7 +330,7 @@ def swa_attention(
     max_seq_len = k_cache.shape[1]
     if num_splits <= 0:
         num_splits = lib.sdv2_swa_attn_default_splits(rows, q_tokens, heads, max_seq_len)
-    need = lib.sdv2_swa_attn_workspace_bytes(rows, q_tokens, heads, max_seq_len, num_splits)
+    need = 0 if static_scratch else lib.sdv2_swa_attn_workspace_bytes(rows, q_tokens, heads, max_seq_len, num_splits)
     if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
         workspace = _workspace(dev, need)
 
@@ -347,7 +354,10 @@ def swa_attention(
         p.mask_block_tokens = int(mask_block_tokens)
         p.chunk_key_start = chunk_key_start.data_ptr()
     with torch.cuda.device(dev):
-        _capi.check(lib.sdv2_swa_attn_fwd(C.byref(p)), "sdv2_swa_attn_fwd")
+        if static_scratch:
+            _capi.check(lib.sdv2_swa_attn_fwd_static(C.byref(p)), "sdv2_swa_attn_fwd_static")
+        else:
+            _capi.check(lib.sdv2_swa_attn_fwd(C.byref(p)), "sdv2_swa_attn_fwd")
     return out
 
 

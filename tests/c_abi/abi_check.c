@@ -80,6 +80,7 @@ int main(void) {
   printf("workspace for that call: %zu bytes\n", sdv2_swa_attn_workspace_bytes(1, 1560, 12, 9360, 0));
   printf("sink-similarity workspace, 1 row, 12 heads, 3 sink frames: %zu bytes\n",
          sdv2_sink_similarity_workspace_bytes(1, 12, 3));
+  expect("attention_static(NULL)", sdv2_swa_attn_fwd_static(NULL), SDV2_ERR_INVALID_ARG);
   expect("event_create(NULL)", sdv2_event_create(NULL), SDV2_ERR_INVALID_ARG);
   expect("copy of nothing", sdv2_copy_bytes(NULL, NULL, 0, NULL), SDV2_OK);
   printf(failures ? "FAILED: %d\n" : "all checks passed\n", failures);

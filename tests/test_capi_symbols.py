@@ -32,7 +32,7 @@ def test_header_constants_match_binding():
     text = open(HEADER).read()
     assert int(re.search(r"#define SDV2_MAX_ROWS (\d+)", text).group(1)) == _capi.MAX_ROWS
     assert int(re.search(r"#define SDV2_HEAD_DIM (\d+)", text).group(1)) == _capi.HEAD_DIM
-    for name in ("INVALID_ARG", "UNSUPPORTED", "OUT_OF_RANGE", "WORKSPACE", "LAUNCH"):
+    for name in ("INVALID_ARG", "UNSUPPORTED", "OUT_OF_RANGE", "WORKSPACE", "LAUNCH", "SCRATCH_LIMIT"):
         val = int(re.search(rf"SDV2_ERR_{name} = (-\d+)", text).group(1))
         assert getattr(_capi, f"SDV2_ERR_{name}") == val
     # struct field order of the binding follows the header
