@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SDV2KV_ABI_VERSION 6
+#define SDV2KV_ABI_VERSION 7
 #define SDV2_HEAD_DIM 128      /* causal_stream_inference.py:99-100 fixes 128 */
 #define SDV2_MAX_ROWS 16       /* rows (B) per sdv2_kv_append_rope call       */
 #define SDV2_MAX_SINK_FRAMES 16 /* sink frames per sdv2_sink_similarity call  */
@@ -126,8 +126,6 @@ typedef struct sdv2_append_params {
   const void* q_norm_weight;   /* device, or NULL (together with k_norm_weight) */
   const void* k_norm_weight;
   float norm_eps;
-  void* timing_start;          /* optional sdv2 timing events (see sdv2_event_create): */
-  void* timing_stop;           /* recorded with the kernel's own dispatch              */
   /* Optional slot chosen on the device: device int64 [B] or NULL.  A value
    * >= 0 (and fitting the cache) replaces dst_start[i]; sdv2_sink_similarity
    * writes it, so that an adaptive sink refresh needs no host round trip
@@ -153,10 +151,6 @@ int sdv2_kv_append_rope(const sdv2_append_params* p);
  * go through `workspace` (size from sdv2_swa_attn_workspace_bytes) and are
  * merged by a second kernel on the same stream.
  * ---------------------------------------------------------------------- */
-#define SDV2_STAGE_ALL 0
-#define SDV2_STAGE_PARTIAL 1
-#define SDV2_STAGE_MERGE 2
-
 typedef struct sdv2_attn_params {
   const void* q;               /* [B,S,H,128] bf16 (roped)                     */
   const void* k_cache;         /* [B,L,H,128] bf16 view of the cache           */
@@ -167,9 +161,6 @@ typedef struct sdv2_attn_params {
   int32_t rows, q_tokens, heads, head_dim;        /* B, S, H, 128              */
   int32_t max_seq_len;                            /* L = k_cache.shape[1]      */
   int32_t num_splits;          /* 0 = choose from the shape                    */
-  int32_t stages;              /* 0 = whole operator; SDV2_STAGE_PARTIAL /     */
-                               /* SDV2_STAGE_MERGE run one of the two kernels  */
-                               /* of a split call (for timing them apart)      */
   float softmax_scale;         /* <= 0 selects 1/sqrt(head_dim)                */
   void* workspace;             /* device scratch, 256-byte aligned             */
   size_t workspace_bytes;
@@ -183,10 +174,6 @@ typedef struct sdv2_attn_params {
    * [chunk_key_start[i] + (t / b + 1) * b, chunk_key_start[i] + S); everything
    * else in the cache is older and stays visible.  0 (or b >= S) = no mask.  */
   int32_t mask_block_tokens;
-  void* timing_start;          /* optional timing events around the attention kernel   */
-  void* timing_stop;
-  void* merge_timing_start;    /* ... and around the merge kernel of a split call      */
-  void* merge_timing_stop;
   const int32_t* chunk_key_start;  /* device int32 [B], each in [0, L - S]; may be */
                                    /* NULL when the mask is off                    */
 } sdv2_attn_params;
@@ -301,32 +288,9 @@ typedef struct sdv2_relayout_params {
   int64_t* dst_local_end_index;
   int64_t global_end_shift;
   void* stream;                /* hipStream_t                                  */
-  void* timing_start;          /* optional timing events                       */
-  void* timing_stop;
 } sdv2_relayout_params;
 
 int sdv2_cache_relayout(const sdv2_relayout_params* p);
-
-/* ------------------------------------------------------------------------
- * Timing events.  No counterpart in the reference: they exist for
- * measurement.  An event handed to a launch through timing_start /
- * timing_stop is recorded in the dispatch of that one kernel (start when the
- * kernel begins to execute, stop when it has finished), so the interval is
- * the kernel's own duration as a profiler reports it, without the gap that
- * separate event records on the stream would add.  sdv2_event_elapsed_ms
- * waits for the stop event.
- * ---------------------------------------------------------------------- */
-int sdv2_event_create(void** event);
-int sdv2_event_destroy(void* event);
-int sdv2_event_elapsed_ms(void* start, void* stop, float* ms);
-
-/* ------------------------------------------------------------------------
- * Plain device-to-device copy of `bytes` bytes with the library's own 16-byte
- * vector kernel.  No counterpart in the reference: it exists so that hardware
- * counters (bytes fetched / written per dispatch) can be scaled against a
- * kernel whose traffic is known exactly.
- * ---------------------------------------------------------------------- */
-int sdv2_copy_bytes(void* dst, const void* src, size_t bytes, void* stream);
 
 #ifdef __cplusplus
 }

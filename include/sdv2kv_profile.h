@@ -1,0 +1,63 @@
+/*
+ * sdv2kv_profile — measurement hooks of libsdv2kv.so.
+ *
+ * Nothing here has a counterpart in the reference and no binding of the path
+ * needs it: these calls exist so that a benchmark can time each kernel of the
+ * path on its own and scale hardware counters.  The operator interface is
+ * include/sdv2kv.h.
+ */
+#ifndef SDV2KV_PROFILE_H
+#define SDV2KV_PROFILE_H
+
+#include "sdv2kv.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* kernels a timing request can name */
+typedef enum sdv2_profile_kernel {
+  SDV2_KERNEL_APPEND = 0,      /* sdv2_kv_append_rope                          */
+  SDV2_KERNEL_ATTENTION = 1,   /* sdv2_swa_attn_fwd: the attention kernel      */
+  SDV2_KERNEL_MERGE = 2,       /* sdv2_swa_attn_fwd: merge of a split call     */
+  SDV2_KERNEL_RELAYOUT = 3,    /* sdv2_cache_relayout                          */
+  SDV2_KERNEL_SINK_SUM = 4,    /* sdv2_sink_similarity: frame sums             */
+  SDV2_KERNEL_SINK_DECIDE = 5, /* sdv2_sink_similarity: decision               */
+  SDV2_KERNEL_COUNT = 6
+} sdv2_profile_kernel;
+
+/* ------------------------------------------------------------------------
+ * Timing events.  An event pair armed with sdv2_profile_time_next is recorded
+ * in the dispatch of the NEXT launch of that kernel made by the calling thread
+ * (start when the kernel begins to execute, stop when it has finished) and
+ * then disarmed, so the interval is the kernel's own duration as a profiler
+ * reports it, without the gap that separate event records on the stream would
+ * add.  NULL, NULL disarms.  sdv2_event_elapsed_ms waits for the stop event.
+ * ---------------------------------------------------------------------- */
+int sdv2_event_create(void** event);
+int sdv2_event_destroy(void* event);
+int sdv2_event_elapsed_ms(void* start, void* stop, float* ms);
+int sdv2_profile_time_next(int kernel, void* start, void* stop);
+
+/* ------------------------------------------------------------------------
+ * Which kernels of a split attention call the calling thread's following
+ * sdv2_swa_attn_fwd calls launch: both (the default), the attention kernel
+ * only (partial results stay in the workspace) or the merge only.  For timing
+ * the two apart over many repetitions; stays in force until set again.
+ * ---------------------------------------------------------------------- */
+#define SDV2_STAGE_ALL 0
+#define SDV2_STAGE_PARTIAL 1
+#define SDV2_STAGE_MERGE 2
+int sdv2_profile_attention_stages(int stages);
+
+/* ------------------------------------------------------------------------
+ * Plain device-to-device copy of `bytes` bytes with the library's own 16-byte
+ * vector kernel, so that hardware counters (bytes fetched / written per
+ * dispatch) can be scaled against a kernel whose traffic is known exactly.
+ * ---------------------------------------------------------------------- */
+int sdv2_copy_bytes(void* dst, const void* src, size_t bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SDV2KV_PROFILE_H */

@@ -1,4 +1,5 @@
-"""ctypes binding of the sdv2kv C ABI (include/sdv2kv.h).
+"""ctypes binding of the sdv2kv C ABI (include/sdv2kv.h; the measurement hooks of
+include/sdv2kv_profile.h at the end).
 
 The shared library is the product: there is no Python or CPU fallback.  When
 it is missing, :func:`lib` raises ImportError with the build command.
@@ -11,7 +12,7 @@ from typing import Optional
 
 LIB_PATH = Path(__file__).resolve().parent / "_lib" / "libsdv2kv.so"
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 HEAD_DIM = 128
 MAX_ROWS = 16
 
@@ -29,7 +30,9 @@ STAGE_ALL, STAGE_PARTIAL, STAGE_MERGE = 0, 1, 2
 DTYPE_BF16 = 0
 DTYPE_F32 = 1
 
-# every symbol include/sdv2kv.h declares
+KERNEL_APPEND, KERNEL_ATTENTION, KERNEL_MERGE, KERNEL_RELAYOUT, KERNEL_SINK_SUM, KERNEL_SINK_DECIDE = range(6)
+
+# every symbol include/sdv2kv.h and include/sdv2kv_profile.h declare
 EXPORTED_SYMBOLS = (
     "sdv2_abi_version",
     "sdv2_status_string",
@@ -44,6 +47,8 @@ EXPORTED_SYMBOLS = (
     "sdv2_event_create",
     "sdv2_event_destroy",
     "sdv2_event_elapsed_ms",
+    "sdv2_profile_time_next",
+    "sdv2_profile_attention_stages",
     "sdv2_copy_bytes",
 )
 
@@ -74,8 +79,6 @@ class AppendParams(C.Structure):
         ("q_norm_weight", C.c_void_p),
         ("k_norm_weight", C.c_void_p),
         ("norm_eps", C.c_float),
-        ("timing_start", C.c_void_p),
-        ("timing_stop", C.c_void_p),
         ("dst_start_override", C.c_void_p),
     ]
 
@@ -88,16 +91,11 @@ class AttnParams(C.Structure):
         ("rows", C.c_int32), ("q_tokens", C.c_int32), ("heads", C.c_int32), ("head_dim", C.c_int32),
         ("max_seq_len", C.c_int32),
         ("num_splits", C.c_int32),
-        ("stages", C.c_int32),
         ("softmax_scale", C.c_float),
         ("workspace", C.c_void_p),
         ("workspace_bytes", C.c_size_t),
         ("stream", C.c_void_p),
         ("mask_block_tokens", C.c_int32),
-        ("timing_start", C.c_void_p),
-        ("timing_stop", C.c_void_p),
-        ("merge_timing_start", C.c_void_p),
-        ("merge_timing_stop", C.c_void_p),
         ("chunk_key_start", C.c_void_p),
     ]
 
@@ -136,7 +134,6 @@ class RelayoutParams(C.Structure):
         ("dst_global_end_index", C.c_void_p), ("dst_local_end_index", C.c_void_p),
         ("global_end_shift", C.c_int64),
         ("stream", C.c_void_p),
-        ("timing_start", C.c_void_p), ("timing_stop", C.c_void_p),
     ]
 
 
@@ -187,6 +184,10 @@ def lib() -> C.CDLL:
     handle.sdv2_event_destroy.argtypes = [C.c_void_p]
     handle.sdv2_event_elapsed_ms.restype = C.c_int
     handle.sdv2_event_elapsed_ms.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]
+    handle.sdv2_profile_time_next.restype = C.c_int
+    handle.sdv2_profile_time_next.argtypes = [C.c_int, C.c_void_p, C.c_void_p]
+    handle.sdv2_profile_attention_stages.restype = C.c_int
+    handle.sdv2_profile_attention_stages.argtypes = [C.c_int]
     handle.sdv2_copy_bytes.restype = C.c_int
     handle.sdv2_copy_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
     if handle.sdv2_abi_version() != ABI_VERSION:

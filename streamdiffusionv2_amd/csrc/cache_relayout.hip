@@ -18,6 +18,7 @@
 #include <stdint.h>
 
 #include "sdv2kv.h"
+#include "sdv2kv_profile.h"
 #include "sdv2kv_internal.h"
 
 namespace {
@@ -119,7 +120,7 @@ extern "C" int sdv2_cache_relayout(const sdv2_relayout_params* p) {
   int64_t blocks = (total + kThreads * kVecsPerThread - 1) / (kThreads * kVecsPerThread);
   if (blocks < 1) blocks = 1;
   if (blocks > 0x7fffffff) return SDV2_ERR_INVALID_ARG;
-  sdv2::launch_timed(cache_relayout_kernel, dim3((unsigned)blocks, (unsigned)p->rows), dim3(kThreads), 0,
-                     static_cast<hipStream_t>(p->stream), p->timing_start, p->timing_stop, a);
+  sdv2::launch_timed(SDV2_KERNEL_RELAYOUT, cache_relayout_kernel, dim3((unsigned)blocks, (unsigned)p->rows),
+                     dim3(kThreads), 0, static_cast<hipStream_t>(p->stream), a);
   return hipGetLastError() == hipSuccess ? SDV2_OK : SDV2_ERR_LAUNCH;
 }

@@ -17,6 +17,7 @@
 #include <type_traits>
 
 #include "sdv2kv.h"
+#include "sdv2kv_profile.h"
 #include "sdv2kv_internal.h"
 #include "rope_device.h"
 
@@ -248,7 +249,6 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
   if (!p->start_frame || (with_kv && !p->dst_start)) return SDV2_ERR_INVALID_ARG;
   if ((p->global_end_index || p->local_end_index) && (!p->new_global_end || !p->new_local_end))
     return SDV2_ERR_INVALID_ARG;
-  if ((p->timing_start == nullptr) != (p->timing_stop == nullptr)) return SDV2_ERR_INVALID_ARG;
   const bool with_norm = p->q_norm_weight != nullptr || p->k_norm_weight != nullptr;
   if (with_norm) {
     // the fused norm covers q and k together, as qkv_fn applies it
@@ -311,11 +311,9 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
     auto launch = [&](auto steps_c) {
       constexpr int kS = decltype(steps_c)::value;
       if (p->dtype == SDV2_BF16)
-        sdv2::launch_timed(kv_append_norm_rope_kernel<uint16_t, kS>, norm_grid, block, 0, stream, p->timing_start,
-                           p->timing_stop, a);
+        sdv2::launch_timed(SDV2_KERNEL_APPEND, kv_append_norm_rope_kernel<uint16_t, kS>, norm_grid, block, 0, stream, a);
       else
-        sdv2::launch_timed(kv_append_norm_rope_kernel<float, kS>, norm_grid, block, 0, stream, p->timing_start,
-                           p->timing_stop, a);
+        sdv2::launch_timed(SDV2_KERNEL_APPEND, kv_append_norm_rope_kernel<float, kS>, norm_grid, block, 0, stream, a);
     };
     const int steps = (p->heads + 3) / 4;
     if (steps <= 4) launch(std::integral_constant<int, 4>{});
@@ -324,7 +322,7 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
     return hipGetLastError() == hipSuccess ? SDV2_OK : SDV2_ERR_LAUNCH;
   }
   auto launch = [&](auto kernel) {
-    sdv2::launch_timed(kernel, grid, block, 0, stream, p->timing_start, p->timing_stop, a);
+    sdv2::launch_timed(SDV2_KERNEL_APPEND, kernel, grid, block, 0, stream, a);
   };
   if (p->dtype == SDV2_BF16) {
     if (!with_kv) launch(kv_append_rope_kernel<uint16_t, true, false>);

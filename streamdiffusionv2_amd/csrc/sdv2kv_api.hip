@@ -4,8 +4,13 @@
 #include <stdint.h>
 
 #include "sdv2kv.h"
+#include "sdv2kv_profile.h"
+#include "sdv2kv_internal.h"
 
 namespace {
+
+thread_local sdv2::TimingPair armed[SDV2_KERNEL_COUNT];
+thread_local int stages_now = SDV2_STAGE_ALL;
 
 __global__ __launch_bounds__(256) void copy16_kernel(uint4* dst, const uint4* src, size_t n16) {
   const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -13,6 +18,28 @@ __global__ __launch_bounds__(256) void copy16_kernel(uint4* dst, const uint4* sr
 }
 
 }  // namespace
+
+sdv2::TimingPair sdv2::take_timing(int kernel) {
+  if (kernel < 0 || kernel >= SDV2_KERNEL_COUNT) return {nullptr, nullptr};
+  const TimingPair t = armed[kernel];
+  armed[kernel] = {nullptr, nullptr};
+  return t;
+}
+
+int sdv2::attention_stages() { return stages_now; }
+
+extern "C" int sdv2_profile_time_next(int kernel, void* start, void* stop) {
+  if (kernel < 0 || kernel >= SDV2_KERNEL_COUNT) return SDV2_ERR_INVALID_ARG;
+  if ((start == nullptr) != (stop == nullptr)) return SDV2_ERR_INVALID_ARG;
+  armed[kernel] = {start, stop};
+  return SDV2_OK;
+}
+
+extern "C" int sdv2_profile_attention_stages(int stages) {
+  if (stages < SDV2_STAGE_ALL || stages > SDV2_STAGE_MERGE) return SDV2_ERR_INVALID_ARG;
+  stages_now = stages;
+  return SDV2_OK;
+}
 
 extern "C" int sdv2_abi_version(void) { return SDV2KV_ABI_VERSION; }
 

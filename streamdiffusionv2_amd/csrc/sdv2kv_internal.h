@@ -8,14 +8,25 @@
 
 namespace sdv2 {
 
-// Launch with the caller's optional timing events attached to the kernel's own
-// dispatch (both or none).
+// Measurement hooks (sdv2kv_profile.h), kept per calling thread in
+// sdv2kv_api.hip: the event pair armed for the next launch of a kernel (taken
+// = disarmed) and the stages a split attention call runs.
+struct TimingPair {
+  void* start;
+  void* stop;
+};
+TimingPair take_timing(int kernel);
+int attention_stages();
+
+// Launch kernel `which` (an sdv2_profile_kernel); when the calling thread has
+// armed timing events for it they are attached to the kernel's own dispatch.
 template <typename Kernel, typename Args>
-inline void launch_timed(Kernel kernel, dim3 grid, dim3 block, uint32_t lds_bytes, hipStream_t stream, void* start,
-                         void* stop, const Args& args) {
-  if (start && stop)
-    hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, static_cast<hipEvent_t>(start),
-                          static_cast<hipEvent_t>(stop), 0, args);
+inline void launch_timed(int which, Kernel kernel, dim3 grid, dim3 block, uint32_t lds_bytes, hipStream_t stream,
+                         const Args& args) {
+  const TimingPair t = take_timing(which);
+  if (t.start && t.stop)
+    hipExtLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, static_cast<hipEvent_t>(t.start),
+                          static_cast<hipEvent_t>(t.stop), 0, args);
   else
     hipLaunchKernelGGL(kernel, grid, block, lds_bytes, stream, args);
 }

@@ -24,6 +24,7 @@
 #include <stdint.h>
 
 #include "sdv2kv.h"
+#include "sdv2kv_profile.h"
 #include "sdv2kv_internal.h"
 #include "rope_device.h"
 
@@ -330,14 +331,15 @@ extern "C" int sdv2_sink_similarity(const sdv2_sink_sim_params* p) {
   const dim3 grid_decide(p->rows);
   // columns per thread of the decision kernel: 2 up to 16 heads, 8 up to 64
   const bool wide = p->heads * 128 > 2 * kDecideThreads;
+  const dim3 decide_block(kDecideThreads);
   if (p->dtype == SDV2_BF16) {
-    hipLaunchKernelGGL(sink_frame_sum_kernel<uint16_t>, grid_mean, block, 0, stream, a);
-    if (wide) hipLaunchKernelGGL((sink_decide_kernel<uint16_t, 8>), grid_decide, dim3(kDecideThreads), 0, stream, a);
-    else hipLaunchKernelGGL((sink_decide_kernel<uint16_t, 2>), grid_decide, dim3(kDecideThreads), 0, stream, a);
+    sdv2::launch_timed(SDV2_KERNEL_SINK_SUM, sink_frame_sum_kernel<uint16_t>, grid_mean, block, 0, stream, a);
+    if (wide) sdv2::launch_timed(SDV2_KERNEL_SINK_DECIDE, sink_decide_kernel<uint16_t, 8>, grid_decide, decide_block, 0, stream, a);
+    else sdv2::launch_timed(SDV2_KERNEL_SINK_DECIDE, sink_decide_kernel<uint16_t, 2>, grid_decide, decide_block, 0, stream, a);
   } else {
-    hipLaunchKernelGGL(sink_frame_sum_kernel<float>, grid_mean, block, 0, stream, a);
-    if (wide) hipLaunchKernelGGL((sink_decide_kernel<float, 8>), grid_decide, dim3(kDecideThreads), 0, stream, a);
-    else hipLaunchKernelGGL((sink_decide_kernel<float, 2>), grid_decide, dim3(kDecideThreads), 0, stream, a);
+    sdv2::launch_timed(SDV2_KERNEL_SINK_SUM, sink_frame_sum_kernel<float>, grid_mean, block, 0, stream, a);
+    if (wide) sdv2::launch_timed(SDV2_KERNEL_SINK_DECIDE, sink_decide_kernel<float, 8>, grid_decide, decide_block, 0, stream, a);
+    else sdv2::launch_timed(SDV2_KERNEL_SINK_DECIDE, sink_decide_kernel<float, 2>, grid_decide, decide_block, 0, stream, a);
   }
   return hipGetLastError() == hipSuccess ? SDV2_OK : SDV2_ERR_LAUNCH;
 }

@@ -47,6 +47,7 @@
 #include <utility>
 
 #include "sdv2kv.h"
+#include "sdv2kv_profile.h"
 #include "sdv2kv_internal.h"
 
 namespace {
@@ -1017,8 +1018,8 @@ int attn_fwd(const sdv2_attn_params* p, void* workspace, size_t workspace_bytes)
   int splits = p->num_splits > 0 ? p->num_splits
                                  : sdv2_swa_attn_default_splits(p->rows, p->q_tokens, p->heads, p->max_seq_len);
   if (splits > 64) return SDV2_ERR_INVALID_ARG;
-  if (p->stages < SDV2_STAGE_ALL || p->stages > SDV2_STAGE_MERGE) return SDV2_ERR_INVALID_ARG;
-  if (p->stages != SDV2_STAGE_ALL && splits == 1) return SDV2_ERR_INVALID_ARG;
+  // measurement hook: a split call can be told to run only one of its two kernels
+  const int stages = splits > 1 ? sdv2::attention_stages() : SDV2_STAGE_ALL;
   if ((int64_t)p->rows * splits > 65535) return SDV2_ERR_INVALID_ARG;
 
   AttnKernelArgs a{};
@@ -1033,9 +1034,6 @@ int attn_fwd(const sdv2_attn_params* p, void* workspace, size_t workspace_bytes)
   const float scale = p->softmax_scale > 0.f ? p->softmax_scale : 0.08838834764831845f;  // 1/sqrt(128)
   a.scale_log2 = scale * kLog2e;
   if (p->mask_block_tokens < 0) return SDV2_ERR_INVALID_ARG;
-  if ((p->timing_start == nullptr) != (p->timing_stop == nullptr) ||
-      (p->merge_timing_start == nullptr) != (p->merge_timing_stop == nullptr))
-    return SDV2_ERR_INVALID_ARG;
   if (p->mask_block_tokens > 0 && p->mask_block_tokens < p->q_tokens) {
     // a block as long as the chunk hides nothing: only shorter blocks switch the mask on
     if (!p->chunk_key_start) return SDV2_ERR_INVALID_ARG;
@@ -1059,7 +1057,7 @@ int attn_fwd(const sdv2_attn_params* p, void* workspace, size_t workspace_bytes)
   const int64_t items = (int64_t)((p->q_tokens + kQTile - 1) / kQTile) * p->heads * p->rows * splits;
   if (items > (1 << 28)) return SDV2_ERR_INVALID_ARG;
   dim3 grid((unsigned)(8 * ((items + 7) / 8)));
-  if (p->stages != SDV2_STAGE_MERGE) {
+  if (stages != SDV2_STAGE_MERGE) {
     // The tile buffers (96 KB) or the epilogue staging (16 KB per wave) exceed the static limit:
     // ask for the dynamic size once per device.
     // The kernel exists twice: the mask inside the chunk costs the plain
@@ -1076,17 +1074,15 @@ int attn_fwd(const sdv2_attn_params* p, void* workspace, size_t workspace_bytes)
       lds_ready[device].store(true, std::memory_order_release);
     }
     if (a.mask_block_tokens > 0)
-      sdv2::launch_timed(swa_attn_fwd_kernel<true>, grid, dim3(kThreads), kLdsBytes, stream, p->timing_start,
-                         p->timing_stop, a);
+      sdv2::launch_timed(SDV2_KERNEL_ATTENTION, swa_attn_fwd_kernel<true>, grid, dim3(kThreads), kLdsBytes, stream, a);
     else
-      sdv2::launch_timed(swa_attn_fwd_kernel<false>, grid, dim3(kThreads), kLdsBytes, stream, p->timing_start,
-                         p->timing_stop, a);
+      sdv2::launch_timed(SDV2_KERNEL_ATTENTION, swa_attn_fwd_kernel<false>, grid, dim3(kThreads), kLdsBytes, stream, a);
     if (hipGetLastError() != hipSuccess) return SDV2_ERR_LAUNCH;
   }
-  if (splits > 1 && p->stages != SDV2_STAGE_PARTIAL) {
+  if (splits > 1 && stages != SDV2_STAGE_PARTIAL) {
     const int64_t nq = (int64_t)p->rows * p->heads * p->q_tokens;
-    sdv2::launch_timed(swa_attn_merge_kernel, dim3((unsigned)((nq + 15) / 16)), dim3(256), 0, stream,
-                       p->merge_timing_start, p->merge_timing_stop, a);
+    sdv2::launch_timed(SDV2_KERNEL_MERGE, swa_attn_merge_kernel, dim3((unsigned)((nq + 15) / 16)), dim3(256), 0, stream,
+                       a);
     if (hipGetLastError() != hipSuccess) return SDV2_ERR_LAUNCH;
   }
   return SDV2_OK;

@@ -293,7 +293,6 @@ def swa_attention(
     num_splits: int = 0,
     softmax_scale: Optional[float] = None,
     workspace: Optional[torch.Tensor] = None,
-    stages: int = _capi.STAGE_ALL,
     chunk_key_start: Optional[torch.Tensor] = None,
     mask_block_tokens: int = 0,
     static_scratch: bool = False,
@@ -343,7 +342,6 @@ def swa_attention(
     p.rows, p.q_tokens, p.heads, p.head_dim = rows, q_tokens, heads, HEAD_DIM
     p.max_seq_len = max_seq_len
     p.num_splits = num_splits
-    p.stages = stages
     p.softmax_scale = float(softmax_scale) if softmax_scale else 0.0
     if need:
         p.workspace = workspace.data_ptr()
@@ -448,16 +446,22 @@ def sink_similarity(
 
 
 class KernelTimer:
-    """A start/stop pair of the library's timing events.  Handed to a launch
-    (``LayerLauncher.set_timers``) it is recorded in that kernel's own
-    dispatch, so :meth:`elapsed_ms` is the kernel's duration as a profiler
-    reports it, without the gap separate stream events add."""
+    """A start/stop pair of the library's timing events (a measurement hook,
+    include/sdv2kv_profile.h).  Armed for a kernel (:meth:`arm`, or
+    ``LayerLauncher.set_timers``) it is recorded in the dispatch of this
+    thread's next launch of that kernel, so :meth:`elapsed_ms` is the kernel's
+    duration as a profiler reports it, without the gap separate stream events
+    add."""
 
     def __init__(self):
         lib = _capi.lib()
         self.start, self.stop = C.c_void_p(), C.c_void_p()
         _capi.check(lib.sdv2_event_create(C.byref(self.start)), "sdv2_event_create")
         _capi.check(lib.sdv2_event_create(C.byref(self.stop)), "sdv2_event_create")
+
+    def arm(self, kernel: int) -> None:
+        """Time this thread's next launch of ``kernel`` (``_capi.KERNEL_*``)."""
+        _capi.check(_capi.lib().sdv2_profile_time_next(kernel, self.start, self.stop), "sdv2_profile_time_next")
 
     def elapsed_ms(self) -> float:
         ms = C.c_float()
@@ -552,6 +556,7 @@ class LayerLauncher:
         self.span = -1
         self.out_stride = None
         self.forced_splits = 0                       # 0 = the library's own choice
+        self.timers = (None, None, None)
 
     def matches(self, q, k, v, kv_cache, freqs_table, qk_norm=None) -> bool:
         if (self._sig(q), self._sig(k), self._sig(v)) != self.in_sig or freqs_table is not self.freqs_table:
@@ -611,16 +616,27 @@ class LayerLauncher:
     def set_timers(self, append: Optional[KernelTimer] = None, attention: Optional[KernelTimer] = None,
                    merge: Optional[KernelTimer] = None) -> None:
         """Attach (or, with None, detach) kernel timers for the next launches."""
-        self.ap.timing_start, self.ap.timing_stop = (append.start, append.stop) if append else (None, None)
-        self.at.timing_start, self.at.timing_stop = (attention.start, attention.stop) if attention else (None, None)
-        self.at.merge_timing_start, self.at.merge_timing_stop = (merge.start, merge.stop) if merge else (None, None)
+        self.timers = (append, attention, merge)
 
     def run_append(self) -> None:
+        if self.timers[0] is not None:
+            self.timers[0].arm(_capi.KERNEL_APPEND)
         _capi.check(self.lib.sdv2_kv_append_rope(self.ap_ref), "sdv2_kv_append_rope")
 
     def run_attention(self, stages: int = _capi.STAGE_ALL) -> None:
-        self.at.stages = stages
-        _capi.check(self.lib.sdv2_swa_attn_fwd(self.at_ref), "sdv2_swa_attn_fwd")
+        """``stages`` other than STAGE_ALL runs one kernel of a split call only
+        (measurement hook; restored before returning)."""
+        if self.timers[1] is not None and stages != _capi.STAGE_MERGE:
+            self.timers[1].arm(_capi.KERNEL_ATTENTION)
+        if self.timers[2] is not None and stages != _capi.STAGE_PARTIAL and self.at.num_splits > 1:
+            self.timers[2].arm(_capi.KERNEL_MERGE)
+        if stages != _capi.STAGE_ALL:
+            _capi.check(self.lib.sdv2_profile_attention_stages(stages), "sdv2_profile_attention_stages")
+        try:
+            _capi.check(self.lib.sdv2_swa_attn_fwd(self.at_ref), "sdv2_swa_attn_fwd")
+        finally:
+            if stages != _capi.STAGE_ALL:
+                self.lib.sdv2_profile_attention_stages(_capi.STAGE_ALL)
 
     def launch(self, q, k, v, start_frames, plan, seq_lens: Optional[torch.Tensor] = None,
                mask_block_tokens: int = 0, dst_start_override: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -715,7 +731,7 @@ def cache_relayout(
         p.global_end_shift = int(global_end_shift)
     p.stream = _stream_ptr(dev)
     if timer is not None:
-        p.timing_start, p.timing_stop = timer.start, timer.stop
+        timer.arm(_capi.KERNEL_RELAYOUT)
     with torch.cuda.device(dev):
         _capi.check(_capi.lib().sdv2_cache_relayout(C.byref(p)), "sdv2_cache_relayout")
 

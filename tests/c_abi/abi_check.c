@@ -7,6 +7,7 @@
 #include <string.h>
 
 #include "sdv2kv.h"
+#include "sdv2kv_profile.h"
 
 static int failures = 0;
 
@@ -73,8 +74,8 @@ int main(void) {
          offsetof(sdv2_attn_params, stream), offsetof(sdv2_attn_params, chunk_key_start));
   printf("layout sdv2_sink_sim_params size=%zu stream=%zu override_rows=%zu\n", sizeof(sdv2_sink_sim_params),
          offsetof(sdv2_sink_sim_params, stream), offsetof(sdv2_sink_sim_params, override_rows));
-  printf("layout sdv2_relayout_params size=%zu stream=%zu timing_stop=%zu\n", sizeof(sdv2_relayout_params),
-         offsetof(sdv2_relayout_params, stream), offsetof(sdv2_relayout_params, timing_stop));
+  printf("layout sdv2_relayout_params size=%zu stream=%zu global_end_shift=%zu\n", sizeof(sdv2_relayout_params),
+         offsetof(sdv2_relayout_params, stream), offsetof(sdv2_relayout_params, global_end_shift));
 
   printf("splits for 1x1560 tokens, 12 heads, 9360 keys: %d\n", sdv2_swa_attn_default_splits(1, 1560, 12, 9360));
   printf("workspace for that call: %zu bytes\n", sdv2_swa_attn_workspace_bytes(1, 1560, 12, 9360, 0));
@@ -82,6 +83,11 @@ int main(void) {
          sdv2_sink_similarity_workspace_bytes(1, 12, 3));
   expect("attention_static(NULL)", sdv2_swa_attn_fwd_static(NULL), SDV2_ERR_INVALID_ARG);
   expect("event_create(NULL)", sdv2_event_create(NULL), SDV2_ERR_INVALID_ARG);
+  expect("time_next(unknown kernel)", sdv2_profile_time_next(SDV2_KERNEL_COUNT, NULL, NULL), SDV2_ERR_INVALID_ARG);
+  expect("time_next(start only)", sdv2_profile_time_next(SDV2_KERNEL_APPEND, &failures, NULL), SDV2_ERR_INVALID_ARG);
+  expect("time_next(disarm)", sdv2_profile_time_next(SDV2_KERNEL_APPEND, NULL, NULL), SDV2_OK);
+  expect("attention_stages(7)", sdv2_profile_attention_stages(7), SDV2_ERR_INVALID_ARG);
+  expect("attention_stages(all)", sdv2_profile_attention_stages(SDV2_STAGE_ALL), SDV2_OK);
   expect("copy of nothing", sdv2_copy_bytes(NULL, NULL, 0, NULL), SDV2_OK);
   printf(failures ? "FAILED: %d\n" : "all checks passed\n", failures);
   return failures ? 1 : 0;
