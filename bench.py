@@ -119,8 +119,7 @@ def gpu_bench(args, w):
         plan = ring.plan_append(cache, path.evict_idx, starts, S, frame_tokens, path.sink_size)
         launcher = path._layer_launcher(q, k, v, cache, table, w.grid)
         launcher.patch(q, k, v, [c // frame_tokens for c in starts], plan, None)
-        split = launcher.at.num_splits > 1
-        t = (ops.KernelTimer(), ops.KernelTimer(), ops.KernelTimer() if split else None)
+        t = (ops.KernelTimer(), ops.KernelTimer())
         launcher.set_timers(*t)
         launcher.run_append()
         launcher.run_attention()
@@ -172,7 +171,6 @@ def gpu_bench(args, w):
     torch.cuda.synchronize()
     t_append = sum(t[0].elapsed_ms() for t in timers) / len(timers)
     t_attn = sum(t[1].elapsed_ms() for t in timers) / len(timers)
-    t_merge = sum(t[2].elapsed_ms() for t in timers if t[2]) / len(timers)
     for t in timers:
         for x in t:
             if x:
@@ -202,7 +200,6 @@ def gpu_bench(args, w):
         "fill_ms": fill_ms,
         "append_ms": t_append,
         "attn_ms": t_attn,
-        "merge_ms": t_merge,
         "splits": splits,
     }
 
@@ -530,7 +527,8 @@ def main():
     tokens = w.rows * w.chunk_tokens
     attn_s = g["attn_ms"] * 1e-3
     achieved_tflops = w.attn_flops() / attn_s / 1e12
-    append_gbs = w.append_bytes(with_q=True) / (g["append_ms"] * 1e-3) / 1e9
+    # the query is rotated inside the attention kernel: the append moves K and V only
+    append_gbs = w.append_bytes(with_q=False) / (g["append_ms"] * 1e-3) / 1e9
     hbm = MEASURED_HBM_BYTES.get(w.name)
     if hbm is not None and hbm["splits"] != g["splits"]:
         hbm = None
@@ -573,10 +571,10 @@ def main():
             "unit": "GB/s",
             "frac": append_gbs / PEAK_HBM_GBS,
             "traffic": hbm["append"] if hbm else None,
-            "bytes_per_launch": w.append_bytes(with_q=True),
+            "bytes_per_launch": w.append_bytes(with_q=False),
             "avg_launch_ms": g["append_ms"],
         },
-        "kernel_ms_per_layer": {"append": g["append_ms"], "attn": g["attn_ms"], "merge": g["merge_ms"]},
+        "kernel_ms_per_layer": {"append": g["append_ms"], "attn": g["attn_ms"]},
     }
     if g["fill_ms"] is not None:
         result["fill_phase_ms_per_chunk"] = [round(x, 4) for x in g["fill_ms"]]

@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SDV2KV_ABI_VERSION 7
+#define SDV2KV_ABI_VERSION 8
 #define SDV2_HEAD_DIM 128      /* causal_stream_inference.py:99-100 fixes 128 */
 #define SDV2_MAX_ROWS 16       /* rows (B) per sdv2_kv_append_rope call       */
 #define SDV2_MAX_SINK_FRAMES 16 /* sink frames per sdv2_sink_similarity call  */
@@ -148,8 +148,18 @@ int sdv2_kv_append_rope(const sdv2_append_params* p);
  * accumulation, bf16 out.
  *
  * Long caches are split over key ranges to fill the 256 CUs; partial results
- * go through `workspace` (size from sdv2_swa_attn_workspace_bytes) and are
- * merged by a second kernel on the same stream.
+ * go through `workspace` (size from sdv2_swa_attn_workspace_bytes) and the
+ * workgroup that finishes a query tile's last range combines them, in the same
+ * launch.  The workspace begins with one ticket word per (row, head, query
+ * tile): it must be ZERO-FILLED ONCE after allocation (hipMemset, or any fill)
+ * before its first use; every call leaves the tickets at zero again, whatever
+ * shape it had, so the same workspace can serve any sequence of calls that do
+ * not overlap in time.
+ *
+ * The query may arrive before RoPE (rope_freqs != NULL): it is then rotated
+ * while it is loaded, with the arithmetic of sdv2_kv_append_rope, so the
+ * append that precedes the call need not write a rotated copy of q
+ * (causal_model.py:253-266 rotates q only to feed it to this operator).
  * ---------------------------------------------------------------------- */
 typedef struct sdv2_attn_params {
   const void* q;               /* [B,S,H,128] bf16 (roped)                     */
@@ -176,6 +186,15 @@ typedef struct sdv2_attn_params {
   int32_t mask_block_tokens;
   const int32_t* chunk_key_start;  /* device int32 [B], each in [0, L - S]; may be */
                                    /* NULL when the mask is off                    */
+  /* Optional RoPE of q inside the call.  rope_freqs = the device table of
+   * sdv2_kv_append_rope (complex128 [rope_freq_rows, 64] as (re, im)), or NULL
+   * when q is already rotated.  The chunk's S tokens are S / (grid_h * grid_w)
+   * whole frames in (f, h, w) row-major order, the first at absolute frame
+   * rope_start_frame[i]; at most SDV2_MAX_ROWS rows.                         */
+  const double* rope_freqs;
+  int32_t rope_freq_rows;
+  int32_t rope_grid_h, rope_grid_w;
+  const int64_t* rope_start_frame; /* host [B]                                     */
 } sdv2_attn_params;
 
 /* number of key-range splits the library would pick for this shape */
@@ -197,10 +216,10 @@ int sdv2_swa_attn_fwd(const sdv2_attn_params* p);
  * that returns SDV2_ERR_SCRATCH_LIMIT and launches nothing (64 MiB covers the
  * Wan 1.3B and 14B shapes at 480p: one row of a 1560-token chunk against six
  * frames).  The call allocates and frees nothing and does not synchronise.
- * Nothing in the scratch has to be cleared between calls (the merge reads only
- * what the same call's attention kernel wrote), but all calls on one GPU share
- * it: two calls that overlap in time on one GPU - different streams, threads
- * or processes' graphs replayed concurrently - race.
+ * The scratch starts out zeroed and every call leaves its ticket words at zero
+ * again, so nothing has to be cleared between calls, but all calls on one GPU
+ * share it: two calls that overlap in time on one GPU - different streams,
+ * threads or graphs replayed concurrently - race.
  * ---------------------------------------------------------------------- */
 #define SDV2_STATIC_SCRATCH_BYTES (64u << 20)
 int sdv2_swa_attn_fwd_static(const sdv2_attn_params* p);

@@ -18,12 +18,11 @@ extern "C" {
 /* kernels a timing request can name */
 typedef enum sdv2_profile_kernel {
   SDV2_KERNEL_APPEND = 0,      /* sdv2_kv_append_rope                          */
-  SDV2_KERNEL_ATTENTION = 1,   /* sdv2_swa_attn_fwd: the attention kernel      */
-  SDV2_KERNEL_MERGE = 2,       /* sdv2_swa_attn_fwd: merge of a split call     */
-  SDV2_KERNEL_RELAYOUT = 3,    /* sdv2_cache_relayout                          */
-  SDV2_KERNEL_SINK_SUM = 4,    /* sdv2_sink_similarity: frame sums             */
-  SDV2_KERNEL_SINK_DECIDE = 5, /* sdv2_sink_similarity: decision               */
-  SDV2_KERNEL_COUNT = 6
+  SDV2_KERNEL_ATTENTION = 1,   /* sdv2_swa_attn_fwd                            */
+  SDV2_KERNEL_RELAYOUT = 2,    /* sdv2_cache_relayout                          */
+  SDV2_KERNEL_SINK_SUM = 3,    /* sdv2_sink_similarity: frame sums             */
+  SDV2_KERNEL_SINK_DECIDE = 4, /* sdv2_sink_similarity: decision               */
+  SDV2_KERNEL_COUNT = 5
 } sdv2_profile_kernel;
 
 /* ------------------------------------------------------------------------
@@ -38,17 +37,6 @@ int sdv2_event_create(void** event);
 int sdv2_event_destroy(void* event);
 int sdv2_event_elapsed_ms(void* start, void* stop, float* ms);
 int sdv2_profile_time_next(int kernel, void* start, void* stop);
-
-/* ------------------------------------------------------------------------
- * Which kernels of a split attention call the calling thread's following
- * sdv2_swa_attn_fwd calls launch: both (the default), the attention kernel
- * only (partial results stay in the workspace) or the merge only.  For timing
- * the two apart over many repetitions; stays in force until set again.
- * ---------------------------------------------------------------------- */
-#define SDV2_STAGE_ALL 0
-#define SDV2_STAGE_PARTIAL 1
-#define SDV2_STAGE_MERGE 2
-int sdv2_profile_attention_stages(int stages);
 
 /* ------------------------------------------------------------------------
  * Plain device-to-device copy of `bytes` bytes with the library's own 16-byte

@@ -12,7 +12,7 @@ from typing import Optional
 
 LIB_PATH = Path(__file__).resolve().parent / "_lib" / "libsdv2kv.so"
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 HEAD_DIM = 128
 MAX_ROWS = 16
 
@@ -25,12 +25,10 @@ SDV2_ERR_LAUNCH = -5
 SDV2_ERR_SCRATCH_LIMIT = -6
 STATIC_SCRATCH_BYTES = 64 << 20
 
-STAGE_ALL, STAGE_PARTIAL, STAGE_MERGE = 0, 1, 2
-
 DTYPE_BF16 = 0
 DTYPE_F32 = 1
 
-KERNEL_APPEND, KERNEL_ATTENTION, KERNEL_MERGE, KERNEL_RELAYOUT, KERNEL_SINK_SUM, KERNEL_SINK_DECIDE = range(6)
+KERNEL_APPEND, KERNEL_ATTENTION, KERNEL_RELAYOUT, KERNEL_SINK_SUM, KERNEL_SINK_DECIDE = range(5)
 
 # every symbol include/sdv2kv.h and include/sdv2kv_profile.h declare
 EXPORTED_SYMBOLS = (
@@ -48,7 +46,6 @@ EXPORTED_SYMBOLS = (
     "sdv2_event_destroy",
     "sdv2_event_elapsed_ms",
     "sdv2_profile_time_next",
-    "sdv2_profile_attention_stages",
     "sdv2_copy_bytes",
 )
 
@@ -97,6 +94,10 @@ class AttnParams(C.Structure):
         ("stream", C.c_void_p),
         ("mask_block_tokens", C.c_int32),
         ("chunk_key_start", C.c_void_p),
+        ("rope_freqs", C.c_void_p),
+        ("rope_freq_rows", C.c_int32),
+        ("rope_grid_h", C.c_int32), ("rope_grid_w", C.c_int32),
+        ("rope_start_frame", C.POINTER(C.c_int64)),
     ]
 
 
@@ -186,8 +187,6 @@ def lib() -> C.CDLL:
     handle.sdv2_event_elapsed_ms.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_float)]
     handle.sdv2_profile_time_next.restype = C.c_int
     handle.sdv2_profile_time_next.argtypes = [C.c_int, C.c_void_p, C.c_void_p]
-    handle.sdv2_profile_attention_stages.restype = C.c_int
-    handle.sdv2_profile_attention_stages.argtypes = [C.c_int]
     handle.sdv2_copy_bytes.restype = C.c_int
     handle.sdv2_copy_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
     if handle.sdv2_abi_version() != ABI_VERSION:

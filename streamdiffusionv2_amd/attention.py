@@ -263,9 +263,14 @@ class RingKVPath:
             # steady-state fast path: launch descriptors are built once per
             # (cache, shape) and only patched per call
             launcher = self._layer_launcher(q, k, v, kv_cache, table, (f, h, w), qk_norm)
-            out = launcher.launch(q, k, v, [c // frame_tokens for c in starts], plan, seq, mask_tokens, override)
+            start_frames = [c // frame_tokens for c in starts]
+            out = launcher.launch(q, k, v, start_frames, plan, seq, mask_tokens, override)
             if return_roped_query:
-                return out, launcher.roped_q.clone()
+                # the attention kernel rotates q on the fly and keeps no copy: the
+                # stand-alone rotation gives the same bits (one arithmetic for both)
+                if launcher.roped_q is not None:
+                    return out, launcher.roped_q.clone()
+                return out, ops.causal_rope_apply(q, [(f, h, w)] * rows, table, torch.tensor(start_frames))
             return out
 
         roped_q = ops.kv_append_rope(

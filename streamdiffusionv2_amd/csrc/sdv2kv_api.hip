@@ -10,7 +10,6 @@
 namespace {
 
 thread_local sdv2::TimingPair armed[SDV2_KERNEL_COUNT];
-thread_local int stages_now = SDV2_STAGE_ALL;
 
 __global__ __launch_bounds__(256) void copy16_kernel(uint4* dst, const uint4* src, size_t n16) {
   const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -26,18 +25,10 @@ sdv2::TimingPair sdv2::take_timing(int kernel) {
   return t;
 }
 
-int sdv2::attention_stages() { return stages_now; }
-
 extern "C" int sdv2_profile_time_next(int kernel, void* start, void* stop) {
   if (kernel < 0 || kernel >= SDV2_KERNEL_COUNT) return SDV2_ERR_INVALID_ARG;
   if ((start == nullptr) != (stop == nullptr)) return SDV2_ERR_INVALID_ARG;
   armed[kernel] = {start, stop};
-  return SDV2_OK;
-}
-
-extern "C" int sdv2_profile_attention_stages(int stages) {
-  if (stages < SDV2_STAGE_ALL || stages > SDV2_STAGE_MERGE) return SDV2_ERR_INVALID_ARG;
-  stages_now = stages;
   return SDV2_OK;
 }
 

@@ -10,13 +10,12 @@ namespace sdv2 {
 
 // Measurement hooks (sdv2kv_profile.h), kept per calling thread in
 // sdv2kv_api.hip: the event pair armed for the next launch of a kernel (taken
-// = disarmed) and the stages a split attention call runs.
+// = disarmed).
 struct TimingPair {
   void* start;
   void* stop;
 };
 TimingPair take_timing(int kernel);
-int attention_stages();
 
 // Launch kernel `which` (an sdv2_profile_kernel); when the calling thread has
 // armed timing events for it they are attached to the kernel's own dispatch.

@@ -12,11 +12,15 @@
 //   CU, two waves per SIMD with 256 registers each; wave w owns the 32-row
 //   block 32w..32w+31.  While one wave of a SIMD is held up (issuing its
 //   global->LDS transfers, at the barrier, waiting for an LDS fragment) the
-//   other keeps the matrix pipe fed; measured 3-6 % faster than four waves of
-//   two blocks each (512 registers, every LDS fragment feeding two MFMAs),
-//   which -DSDV2_FOUR_WAVES still builds.  Keys stream through LDS in tiles of
+//   other keeps the matrix pipe fed.  Keys stream through LDS in tiles of
 //   64 (K 16 KB + V 16 KB), three buffers each, filled two tiles ahead by
 //   global->LDS transfers that never touch registers.
+//
+//   Long caches are split over key ranges so that the grid fills the chip.
+//   Every workgroup of a split call leaves its (normalised output, log-sum-exp)
+//   in the workspace and takes a ticket; the workgroup that draws the last
+//   ticket of a (row, head, query tile) combines all ranges and writes the
+//   result, so a split call is still one launch.
 //
 // Matrix layout (v_mfma_f32_32x32x16_bf16, D = A(32x16) * B(16x32) + C):
 //   S^T = K Q^T   A = K tile rows (ds_read_b128), B = Q, in registers for the
@@ -27,13 +31,15 @@
 //   In both products a lane owns ONE query per block (column lane%32), so the
 //   softmax statistics are per-lane scalars.
 //
-// Softmax.  exp2 of the scaled scores is taken without subtracting a running
-// maximum: the weights stay in fp32 / bf16 range as long as the scaled scores
-// stay within about +-100 in log2 units, which every sane attention input
-// does, and the result is mathematically the same.  Each wave checks its row
-// sums after its last tile; if any left [2^-100, 2^100] (or is NaN) the
-// workgroup throws the result away and recomputes with the
-// conventional running-maximum recurrence (slow, exact for any finite input).
+// Softmax.  exp2 of the scaled scores is taken against a FIXED reference per
+// query row, the largest score among the first 32 keys of the workgroup's
+// range, instead of a running maximum: nothing is ever rescaled, and the
+// weights stay in fp32 / bf16 range as long as no later score exceeds that
+// reference by about 100 in log2 units (69 in natural units).  Each wave checks
+// its row sums after its last tile; a wave that finds one outside [2^-100,
+// 2^100] (or NaN) throws its block away and recomputes it with the
+// conventional running-maximum recurrence (slower, exact for any finite
+// input) while the other waves only keep the tiles coming.
 //
 // LDS tile layout: row r (key) holds sixteen 16-byte chunks; chunk c is stored
 // at position c ^ g(r), g(r) = ((r & 3) << 2) | ((r >> 2) & 3).  That makes the
@@ -49,6 +55,7 @@
 #include "sdv2kv.h"
 #include "sdv2kv_profile.h"
 #include "sdv2kv_internal.h"
+#include "rope_device.h"
 
 namespace {
 
@@ -58,23 +65,15 @@ typedef __attribute__((ext_vector_type(4))) short s16x4;
 typedef __attribute__((ext_vector_type(8))) short s16x8;
 typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
-typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
 typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
 typedef __attribute__((address_space(3))) char lds_char;
+typedef __attribute__((address_space(3))) int lds_int;
 
 constexpr int kD = SDV2_HEAD_DIM;           // 128
-#ifndef SDV2_FOUR_WAVES
-constexpr int kWaves = 8;                   // two waves per SIMD
-constexpr int kQB = 1;                      // 32-row query blocks per wave
-#define SDV2_Q_REG "a"                      // 256 registers per wave, at most 128 of them VGPRs: Q lives beside O
-#else
-#define SDV2_Q_REG "v"
-constexpr int kWaves = 4;
-constexpr int kQB = 2;                      // 32-row query blocks per wave
-#endif
+constexpr int kWaves = 8;                   // two waves per SIMD, one 32-row query block each
 constexpr int kThreads = kWaves * 64;
 // The global->LDS transfers of a tile are issued by the first wave of every
 // SIMD only (waves 0-3).  A wave is held while its transfers queue up; with all
@@ -83,17 +82,23 @@ constexpr int kThreads = kWaves * 64;
 // 0.5-1.5 % faster; two or one issuing waves fall far behind the rest).
 constexpr int kIssuers = 4;
 constexpr int kPieces = 16 / kIssuers;      // global->LDS instructions per issuing wave and matrix tile
-constexpr int kQRowsPerWave = 32 * kQB;
-constexpr int kQTile = kWaves * kQRowsPerWave;   // 256
+constexpr int kQBlock = 32;                 // query rows per wave
+constexpr int kQTile = kWaves * kQBlock;    // 256
 constexpr int kKTile = 64;
-constexpr int kTileBytes = kKTile * kD * 2;      // 16 KB per matrix
+constexpr int kTileBytes = kKTile * kD * 2; // 16 KB per matrix
 constexpr int kStages = 3;
-constexpr int kStageBytes = 16384;           // epilogue staging per wave: 32 rows x 512 B
+constexpr int kStageBytes = 16384;          // epilogue staging per wave: 32 rows x 512 B
 constexpr int kLdsBytes = 2 * kStages * kTileBytes > kWaves * kStageBytes ? 2 * kStages * kTileBytes
                                                                          : kWaves * kStageBytes;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kCuSlots = 256;               // one workgroup per CU
 constexpr int kMaxDevices = 64;
+constexpr int kPartBlockHalves = kQBlock * kD;   // one block's partial output: 32 x 128 fp16 = 8 KB
+// The ticket words of a split call sit in a region of FIXED size at the head of
+// the workspace, whatever the shape: a region that grew with the shape would
+// overlap, for a larger call, what an earlier smaller call left of its partial
+// results, and tickets must be zero when a call starts.
+constexpr int kMaxTickets = 16384;               // (row, head, query tile) groups of a split call
 
 // LDS map: kStages K tile buffers, then kStages V tile buffers.  The DS
 // instructions carry a 16-bit offset, so V fragment addresses are kept
@@ -115,9 +120,18 @@ struct AttnKernelArgs {
   float scale_log2;            // softmax_scale * log2(e)
   int32_t mask_block_tokens;   // 0 = no mask inside the chunk
   const int32_t* chunk_start;  // device [rows]: cache position of the chunk's own first key
-  uint16_t* part_o;            // [split][row][head][q][128] fp16: normalised output / row scale
-  float* part_lse;             // [split][row][head][q]      log2 sum exp
-  float* part_scale;           // [split][row][head][q]      largest magnitude of the normalised row
+  // Split calls.  Partial results are kept per 32-row query block in the order
+  // the registers hold them (see store_partial), q_blocks = ceil(q_tokens / 32).
+  int32_t q_blocks;
+  int32_t* tickets;            // [row][head][query tile], zero between calls
+  uint16_t* part_o;            // [split][row][head][block][8 KB] fp16: normalised output / row scale
+  float* part_lse;             // [split][row][head][block][32]   log2 sum exp
+  float* part_scale;           // [split][row][head][block][32]   largest magnitude of the normalised row
+  // Rotation of the queries inside the kernel (q is then the chunk's query
+  // BEFORE RoPE): the complex128 table, or null when q arrives rotated.
+  const double2* freqs;
+  int32_t grid_w, frame_tokens, split_t, split_h;
+  int64_t start_frame[SDV2_MAX_ROWS];
 };
 
 __device__ __forceinline__ int swz(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
@@ -196,7 +210,8 @@ __device__ __forceinline__ void pin(uint32_t& x) { asm volatile("" : "+v"(x)); }
 // compiler keeps every MFMA accumulator in the accumulation registers, but the
 // scores feed the vector ALU (which cannot read those) while the output tile
 // never does until the epilogue; naming the register class per product puts S
-// in VGPRs and O in AGPRs.  `kPending` is the s_waitcnt that makes the A
+// in VGPRs and O (with the Q fragments beside it: at 256 registers per wave at
+// most 128 are VGPRs) in AGPRs.  `kPending` is the s_waitcnt that makes the A
 // fragment valid (reads issued after it that may still be in flight); -1 = the
 // fragment was already waited for.  Nothing here is covered by the compiler's
 // hazard tracking: S is read by the vector ALU a full slot after its last
@@ -206,17 +221,17 @@ template <int kPending>
 __device__ __forceinline__ void mfma_s_first(f32x16& d, const u32x4& a, const bf16x8& b) {
   if constexpr (kPending >= 0)
     asm volatile("s_waitcnt lgkmcnt(%3)\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0"
-                 : "=&v"(d) : "v"(a), SDV2_Q_REG(b), "n"(kPending));
+                 : "=&v"(d) : "v"(a), "a"(b), "n"(kPending));
   else
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), SDV2_Q_REG(b));
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
 }
 template <int kPending>
 __device__ __forceinline__ void mfma_s(f32x16& d, const u32x4& a, const bf16x8& b) {
   if constexpr (kPending >= 0)
     asm volatile("s_waitcnt lgkmcnt(%3)\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0"
-                 : "+v"(d) : "v"(a), SDV2_Q_REG(b), "n"(kPending));
+                 : "+v"(d) : "v"(a), "a"(b), "n"(kPending));
   else
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), SDV2_Q_REG(b));
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
 }
 template <int kPending>
 __device__ __forceinline__ void mfma_o(f32x16& d, const u32x4& a, const u32x4& b) {
@@ -270,6 +285,58 @@ __device__ __forceinline__ void issue_matrix_tile(const char* base, uint32_t tok
   }
 }
 
+// ---------------------------------------------------------------------------
+// Partial results travel between workgroups that may sit on different XCDs,
+// each behind its own L2.  Fences would make that safe by writing back and
+// invalidating a whole L2 per workgroup (measured: 13 us per workgroup, and the
+// K / V lines the neighbours are streaming go with it).  Instead every access
+// to a partial result is itself device-coherent, as a relaxed atomic access of
+// agent scope is (the sc1 scope bit: the store writes through to memory, the
+// load does not hit in a stale line), and the ticket orders them: a workgroup
+// draws its ticket only after its stores have been acknowledged (vmcnt(0),
+// barrier), and the last one reads only after it has drawn.  The 16-byte
+// accesses have no atomic spelling in the language, so they are asm (8-byte
+// atomics were measured 4 % of the whole kernel slower).
+// ---------------------------------------------------------------------------
+__device__ __forceinline__ void store_coherent_x4(void* base, const u32x4& w0, const u32x4& w1, const u32x4& w2,
+                                                  const u32x4& w3) {
+  asm volatile(
+      "global_store_dwordx4 %0, %1, off sc1\n\t"
+      "global_store_dwordx4 %0, %2, off offset:1024 sc1\n\t"
+      "global_store_dwordx4 %0, %3, off offset:2048 sc1\n\t"
+      "global_store_dwordx4 %0, %4, off offset:3072 sc1"
+      :
+      : "v"(base), "v"(w0), "v"(w1), "v"(w2), "v"(w3)
+      : "memory");
+}
+// One block's partial output as this lane holds it: eight 16-byte pieces 1 KB
+// apart.  Issue and wait are ONE asm statement: between a load's issue and its
+// return the compiler believes the destination registers hold the value, and
+// is free to copy them elsewhere and reuse them - as an address, say - for the
+// load to overwrite when it lands.
+__device__ __forceinline__ void load_coherent_x8(const char* base, u32x4 (&w)[8]) {
+  asm volatile(
+      "global_load_dwordx4 %0, %8, off sc1\n\t"
+      "global_load_dwordx4 %1, %8, off offset:1024 sc1\n\t"
+      "global_load_dwordx4 %2, %8, off offset:2048 sc1\n\t"
+      "global_load_dwordx4 %3, %8, off offset:3072 sc1\n\t"
+      "global_load_dwordx4 %4, %9, off sc1\n\t"
+      "global_load_dwordx4 %5, %9, off offset:1024 sc1\n\t"
+      "global_load_dwordx4 %6, %9, off offset:2048 sc1\n\t"
+      "global_load_dwordx4 %7, %9, off offset:3072 sc1\n\t"
+      "s_waitcnt vmcnt(0)"
+      : "=&v"(w[0]), "=&v"(w[1]), "=&v"(w[2]), "=&v"(w[3]), "=&v"(w[4]), "=&v"(w[5]), "=&v"(w[6]), "=&v"(w[7])
+      : "v"(base), "v"(base + 4096)
+      : "memory");
+}
+__device__ __forceinline__ void store_coherent(float* p, float x) {
+  __hip_atomic_store(reinterpret_cast<uint32_t*>(p), __float_as_uint(x), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_coherent(const float* p) {
+  return __uint_as_float(
+      __hip_atomic_load(reinterpret_cast<const uint32_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+
 // The compiler does not know that the asm MFMAs are still in flight when the
 // asm statement retires, so wherever code it generates may touch S or O right
 // after a slot (register moves at control-flow joins, the epilogue) the matrix
@@ -278,29 +345,22 @@ __device__ __forceinline__ void issue_matrix_tile(const char* base, uint32_t tok
 // drains at the ends of sibling branches are merged into one AFTER the join,
 // behind the very moves they are meant to precede.
 template <int kTag>
-__device__ __forceinline__ void mfma_drain(f32x16 (&oacc)[kQB][4], f32x16 (&s)[2][kQB]) {
-  if constexpr (kQB == 2) {
-    asm volatile("s_nop 15\n\ts_nop 15 ; matrix pipe drained, site %12"
-                 : "+a"(oacc[0][0]), "+a"(oacc[0][1]), "+a"(oacc[0][2]), "+a"(oacc[0][3]), "+a"(oacc[kQB - 1][0]),
-                   "+a"(oacc[kQB - 1][1]), "+a"(oacc[kQB - 1][2]), "+a"(oacc[kQB - 1][3]), "+v"(s[0][0]),
-                   "+v"(s[0][kQB - 1]), "+v"(s[1][0]), "+v"(s[1][kQB - 1])
-                 : "n"(kTag));
-  } else {
-    asm volatile("s_nop 15\n\ts_nop 15 ; matrix pipe drained, site %6"
-                 : "+a"(oacc[0][0]), "+a"(oacc[0][1]), "+a"(oacc[0][2]), "+a"(oacc[0][3]), "+v"(s[0][0]), "+v"(s[1][0])
-                 : "n"(kTag));
-  }
+__device__ __forceinline__ void mfma_drain(f32x16 (&oacc)[4], f32x16 (&s)[2]) {
+  asm volatile("s_nop 15\n\ts_nop 15 ; matrix pipe drained, site %6"
+               : "+a"(oacc[0]), "+a"(oacc[1]), "+a"(oacc[2]), "+a"(oacc[3]), "+v"(s[0]), "+v"(s[1])
+               : "n"(kTag));
 }
 
 struct LaneConst {
   uint32_t k_addr[8];     // K fragment of d-step ks: key row lane%32 of a 32-key block
   uint32_t v_addr[4][2];  // V^T fragment of d block db, key sub-quad j, within a 16-key step
   float c2;               // softmax scale * log2(e)
+  float neg_ref;          // minus the row's exponent reference, in log2 units (0 until it is chosen)
   int hf;                 // lane / 32
   // block-causal mask inside the chunk: keys [m_lo, m_hi) are the chunk's own
   // later blocks, hidden from this lane's query; [wg_m_lo, m_hi) is the union
   // over the workgroup's queries (wave-uniform).  Empty when the mask is off.
-  int m_lo[kQB];
+  int m_lo;
   int m_hi;
   int wg_m_lo;
 };
@@ -316,9 +376,9 @@ __device__ __forceinline__ void mask_block(f32x16& s, int key0, int seq, int hf,
 // ---------------------------------------------------------------------------
 // One pipeline slot of the fast pass.  Keys advance in blocks of 32; block j
 // goes through
-//   S(j)  = K_j Q^T            8 K fragments x kQB query blocks MFMAs
-//   SM(j) = exp2(scale * S)    VALU only, kQB x 16 scores per lane
-//   PV(j) = O^T += V_j^T P_j^T 8 V fragments x kQB query blocks MFMAs
+//   S(j)  = K_j Q^T            8 K fragments, one MFMA each
+//   SM(j) = exp2(scale * S - reference)   VALU only, 16 scores per lane
+//   PV(j) = O^T += V_j^T P_j^T 8 V fragments, one MFMA each
 // and slot j runs S(j+1), SM(j) and PV(j-1) together: MFMAs of the two
 // products alternate (consecutive MFMAs never share an accumulator) and the
 // softmax instructions of block j are dealt out between them, so the matrix
@@ -327,19 +387,15 @@ __device__ __forceinline__ void mask_block(f32x16& s, int key0, int seq, int hf,
 // pure register naming.
 // ---------------------------------------------------------------------------
 template <bool kMask, int kPar, int kKOff, int kVOff, bool kDoS, bool kDoPV, bool kDoSM>
-__device__ __forceinline__ void slot(const LaneConst& c, const bf16x8 (&qf)[kQB][8], f32x16 (&s)[2][kQB],
-                                     u32x4 (&p)[2][kQB][2], f32x16 (&oacc)[kQB][4], float (&l)[kQB],
-                                     int key0, int key_end) {
-  // Fragment pairs are requested this many groups early.  With a second wave on
-  // the SIMD to cover the wait, one group ahead is enough and measured 2-3 %
-  // faster than two (fewer fragments in flight); none ahead is 4 % slower.
-#ifndef SDV2_AHEAD
-#define SDV2_AHEAD (kQB == 1 ? 1 : 2)
-#endif
-  constexpr int kAhead = SDV2_AHEAD;
+__device__ __forceinline__ void slot(const LaneConst& c, const bf16x8 (&qf)[8], f32x16 (&s)[2], u32x4 (&p)[2][2],
+                                     f32x16 (&oacc)[4], float& l, int key0, int key_end) {
+  // Fragment pairs are requested one group early: with a second wave on the
+  // SIMD to cover the wait that is enough and measured 2-3 % faster than two
+  // (fewer fragments in flight); none ahead is 4 % slower.
+  constexpr int kAhead = 1;
   u32x4 kfrag[8], vfrag[8];
-  f32x16 (&s_cur)[kQB] = s[kPar];
-  f32x16 (&s_nxt)[kQB] = s[kPar ^ 1];
+  f32x16& s_cur = s[kPar];
+  f32x16& s_nxt = s[kPar ^ 1];
 
   auto request = [&](auto ic) {
     constexpr int g = decltype(ic)::value;
@@ -370,33 +426,24 @@ __device__ __forceinline__ void slot(const LaneConst& c, const bf16x8 (&qf)[kQB]
       masked = masked > into_hidden ? masked : into_hidden;
     }
     asm volatile("" : "+s"(masked));
-    if (masked > 0) {
-#pragma unroll
-      for (int qb = 0; qb < kQB; ++qb)
-        mask_block(s_cur[qb], key0, key_end, c.hf, kMask ? c.m_lo[qb] : 0x7fffffff, kMask ? c.m_hi : 0);
-    }
+    if (masked > 0) mask_block(s_cur, key0, key_end, c.hf, kMask ? c.m_lo : 0x7fffffff, kMask ? c.m_hi : 0);
   }
   __builtin_amdgcn_sched_barrier(0);
 
   // A wave issues in order: a vector instruction only overlaps an MFMA if it
   // follows it in the stream, and it stalls the stream if it needs the result
   // of the instruction just before it.  So every MFMA is followed by a few
-  // softmax instructions that are independent of each other: the 16 kQB scores
+  // softmax instructions that are independent of each other: the 16 scores
   // of block j flow through scale -> exp2 -> pack + row sum one step apart.
-  // Score t belongs to group g = t / (2 kQB): query block (t % (2 kQB)) / 2,
-  // accumulator register 2g + t%2.
-  constexpr int kSPG = 2 * kQB;        // steps (= MFMAs) per fragment group: S of each block, PV of each block
-  constexpr int kSteps = 8 * kSPG;
+  // Step t runs the S MFMA (t even) or the PV MFMA (t odd) of fragment group
+  // t / 2 and handles score t = accumulator register t.
+  constexpr int kSteps = 16;
   float scaled[kSteps + 1], weight[kSteps + 1];
-  auto score = [&](auto tc) -> float {
-    constexpr int t = decltype(tc)::value;
-    return s_cur[(t % kSPG) >> 1][2 * (t / kSPG) + (t & 1)];
-  };
   auto softmax_step = [&](auto tc) {
-    constexpr int t = decltype(tc)::value;      // 0..33: stage 1 of score t, stage 2 of t-1, stage 3 of t-2
+    constexpr int t = decltype(tc)::value;      // 0..17: stage 1 of score t, stage 2 of t-1, stage 3 of t-2
     if constexpr (kDoSM) {
       if constexpr (t < kSteps) {
-        scaled[t] = score(tc) * c.c2;
+        scaled[t] = __builtin_fmaf(s_cur[t], c.c2, c.neg_ref);
         pin(scaled[t]);
       }
       if constexpr (t >= 1 && t - 1 < kSteps) {
@@ -404,33 +451,30 @@ __device__ __forceinline__ void slot(const LaneConst& c, const bf16x8 (&qf)[kQB]
         pin(weight[t - 1]);
       }
       if constexpr (t >= 2 && t - 2 < kSteps && ((t - 2) & 1) == 1) {
-        constexpr int u = t - 2, g = u / kSPG, qb = (u % kSPG) >> 1;
+        constexpr int u = t - 2, g = u / 2;
         uint32_t packed = pack_bf16x2(weight[u - 1], weight[u]);
-        l[qb] = add_bf16_pair(packed, l[qb]);
+        l = add_bf16_pair(packed, l);
         pin(packed);
-        pin(l[qb]);
-        p[kPar][qb][g >> 2][g & 3] = packed;
+        pin(l);
+        p[kPar][g >> 2][g & 3] = packed;
       }
     }
   };
 
   static_for<kSteps>([&](auto tc) {
     constexpr int t = decltype(tc)::value;
-    constexpr int g = t / kSPG, i = t % kSPG;
+    constexpr int g = t / 2, i = t % 2;
     constexpr int later = (g + kAhead < 8 ? kAhead : 7 - g) * kPerGroup;   // reads of later groups in flight
     constexpr int kk = g >> 2, db = g & 3;
     if constexpr (i == 0 && g + kAhead < 8) request(std::integral_constant<int, g + kAhead>{});
 
-    if constexpr (i < kQB && kDoS) {
-      // the first MFMA on a fragment waits for it; the K fragment is followed by this group's two V reads
-      constexpr int pending = i == 0 ? later + (kDoPV ? 2 : 0) : -1;
-      if constexpr (g == 0) mfma_s_first<pending>(s_nxt[i], kfrag[g], qf[i][g]);
-      else mfma_s<pending>(s_nxt[i], kfrag[g], qf[i][g]);
+    if constexpr (i == 0 && kDoS) {
+      // the K fragment is followed by this group's two V reads
+      constexpr int pending = later + (kDoPV ? 2 : 0);
+      if constexpr (g == 0) mfma_s_first<pending>(s_nxt, kfrag[g], qf[g]);
+      else mfma_s<pending>(s_nxt, kfrag[g], qf[g]);
     }
-    if constexpr (i >= kQB && kDoPV) {
-      constexpr int qb = i - kQB;
-      mfma_o<(qb == 0 ? later : -1)>(oacc[qb][db], vfrag[g], p[kPar ^ 1][qb][kk]);
-    }
+    if constexpr (i == 1 && kDoPV) mfma_o<later>(oacc[db], vfrag[g], p[kPar ^ 1][kk]);
 
     softmax_step(tc);
     __builtin_amdgcn_sched_barrier(0);
@@ -440,34 +484,42 @@ __device__ __forceinline__ void slot(const LaneConst& c, const bf16x8 (&qf)[kQB]
 }
 
 // ---------------------------------------------------------------------------
-// Exact pass: conventional online softmax with a running maximum, one 64-key
-// tile at a time, nothing overlapped.  Only reached when the fast pass saw a
-// row sum leave the safe range, so its speed does not matter.
+// Exact pass: conventional online softmax with a running maximum over the
+// workgroup's key range, tiles double-buffered.  Every wave keeps the tiles
+// coming and meets the barriers; only the waves whose fast result was unsafe
+// (`compute`) redo their block.
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ void exact_pass(const AttnKernelArgs& a, const LaneConst& c, const bf16x8 (&qf)[kQB][8],
-                                        f32x16 (&oacc)[kQB][4], float (&m_run)[kQB], float (&l_run)[kQB],
-                                        const char* kbase, const char* vbase, uint32_t k_tok_bytes,
-                                        uint32_t v_tok_bytes, const uint32_t (&k_ld)[kPieces], const uint32_t (&v_ld)[kPieces],
-                                        int tile_begin, int n, int seq, uint32_t lds_addr0, lds_char* lds,
-                                        int wave_u, int lane) {
-#pragma unroll
-  for (int qb = 0; qb < kQB; ++qb) {
-    m_run[qb] = -INFINITY;
-    l_run[qb] = 0.f;
+__device__ __forceinline__ void exact_pass(const LaneConst& c, const bf16x8 (&qf)[8], f32x16 (&oacc)[4], float& m_run,
+                                           float& l_run, bool compute, const char* kbase, const char* vbase,
+                                           uint32_t k_tok_bytes, uint32_t v_tok_bytes, const uint32_t (&k_ld)[kPieces],
+                                           const uint32_t (&v_ld)[kPieces], int tile_begin, int n, int seq,
+                                           uint32_t lds_addr0, lds_char* lds, int wave_u, int lane) {
+  if (compute) {
+    m_run = -INFINITY;
+    l_run = 0.f;
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[qb][db][i] = 0.f;
+      for (int i = 0; i < 16; ++i) oacc[db][i] = 0.f;
   }
+  auto issue = [&](int T) {
+    const int key0 = (tile_begin + T) * kKTile;
+    issue_matrix_tile(kbase, k_tok_bytes, k_ld, key0, seq, lds_addr0 + kLdsK(T & 1), wave_u, lane);
+    issue_matrix_tile(vbase, v_tok_bytes, v_ld, key0, seq, lds_addr0 + kLdsV(T & 1), wave_u, lane);
+  };
+  __syncthreads();       // everyone is done with the buffers of the fast pass
+  issue(0);
   for (int T = 0; T < n; ++T) {
     const int key0 = (tile_begin + T) * kKTile;
-    __syncthreads();     // everyone is done with the previous tile
-    issue_matrix_tile(kbase, k_tok_bytes, k_ld, key0, seq, lds_addr0 + kLdsK(0), wave_u, lane);
-    issue_matrix_tile(vbase, v_tok_bytes, v_ld, key0, seq, lds_addr0 + kLdsV(0), wave_u, lane);
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();
-#pragma unroll
-    for (int qb = 0; qb < kQB; ++qb) {
+    const int kb_off = kLdsK(T & 1), vb_off = kLdsVRel(T & 1);
+    if (T + 1 < n) {
+      issue(T + 1);      // into the buffer tile T - 1 left at the barrier that ended the last trip
+      __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kPieces));
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    }
+    __syncthreads();     // tile T has landed for every wave
+    if (compute) {
       f32x16 sacc[2];
 #pragma unroll
       for (int kb = 0; kb < 2; ++kb) {
@@ -476,11 +528,11 @@ __device__ __forceinline__ void exact_pass(const AttnKernelArgs& a, const LaneCo
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
           const bf16x8 kf = *reinterpret_cast<__attribute__((address_space(3))) const bf16x8*>(
-              lds + (c.k_addr[ks] - lds_addr0) + kLdsK(0) + kb * 32 * 256);
-          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[qb][ks], sacc[kb], 0, 0, 0);
+              lds + (c.k_addr[ks] - lds_addr0) + kb_off + kb * 32 * 256);
+          sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc[kb], 0, 0, 0);
         }
         if (key0 + kb * 32 + 32 > seq || (key0 + kb * 32 + 32 > c.wg_m_lo && key0 + kb * 32 < c.m_hi))
-          mask_block(sacc[kb], key0 + kb * 32, seq, c.hf, c.m_lo[qb], c.m_hi);
+          mask_block(sacc[kb], key0 + kb * 32, seq, c.hf, c.m_lo, c.m_hi);
       }
       float mloc = sacc[0][0];
 #pragma unroll
@@ -488,11 +540,11 @@ __device__ __forceinline__ void exact_pass(const AttnKernelArgs& a, const LaneCo
 #pragma unroll
         for (int i = 0; i < 16; ++i) mloc = fmaxf(mloc, sacc[kb][i]);
       mloc = half_max(mloc);
-      const float m_new = fmaxf(m_run[qb], mloc);
+      const float m_new = fmaxf(m_run, mloc);
       // -inf only while every key so far was masked for this query: then nothing has been summed yet
-      const float alpha = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f((m_run[qb] - m_new) * c.c2);
+      const float alpha = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f((m_run - m_new) * c.c2);
       const float mc = m_new == -INFINITY ? 0.0f : m_new * c.c2;
-      m_run[qb] = m_new;
+      m_run = m_new;
       float psum = 0.f;
       bf16x8 pf[2][2];
 #pragma unroll
@@ -509,24 +561,60 @@ __device__ __forceinline__ void exact_pass(const AttnKernelArgs& a, const LaneCo
           }
           pf[kb][st] = pk.v;
         }
-      l_run[qb] = l_run[qb] * alpha + psum;
+      l_run = l_run * alpha + psum;
 #pragma unroll
       for (int db = 0; db < 4; ++db) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) oacc[qb][db][i] *= alpha;
+        for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
           const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(
-              lds + (c.v_addr[db][0] - lds_addr0) + kk * 16 * 256));
+              lds + (c.v_addr[db][0] - lds_addr0) + vb_off + kk * 16 * 256));
           const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(
-              lds + (c.v_addr[db][1] - lds_addr0) + kk * 16 * 256));
+              lds + (c.v_addr[db][1] - lds_addr0) + vb_off + kk * 16 * 256));
           const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          oacc[qb][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both),
-                                                                 pf[kk >> 1][kk & 1], oacc[qb][db], 0, 0, 0);
+          oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf[kk >> 1][kk & 1],
+                                                              oacc[db], 0, 0, 0);
         }
       }
     }
+    __syncthreads();     // tile T's buffer is free for tile T + 2
   }
+}
+
+// This lane's query row as the B operand of S^T = K Q^T: d-step ks takes the
+// 8 elements 16 ks + 8 (lane / 32) of the row.  With a RoPE table the row is
+// the query before rotation and is rotated here, in the arithmetic of the
+// append kernel (IEEE double, no fused multiply-add, double -> float -> bf16),
+// so the kernel sees bit for bit the Q' the append would have stored.
+struct QueryRope {
+  const double2* freqs;        // null: the query arrives rotated
+  int64_t start_frame;         // of this cache row
+  int32_t grid_w, frame_tokens, split_t, split_h;
+};
+
+__device__ __forceinline__ void load_query(const QueryRope& rope, const uint16_t* qp, int token, int hf,
+                                           bf16x8 (&qf)[8]) {
+  if (rope.freqs == nullptr) {
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) qf[ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
+  } else {
+    const int fi = token / rope.frame_tokens;
+    const int rem = token - fi * rope.frame_tokens;
+    const int hi = rem / rope.grid_w;
+    const int wi = rem - hi * rope.grid_w;
+    const int64_t frame = rope.start_frame + fi;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      double2 cs[4];
+      sdv2::load_rotation(rope.freqs, kD / 2, rope.split_t, rope.split_h, 2 * ks + hf, frame, hi, wi, cs);
+      const sdv2::Vec8<uint16_t> y = sdv2::rotate(sdv2::Vec8<uint16_t>::load(qp + 16 * ks), cs);
+      qf[ks] = __builtin_bit_cast(bf16x8, y.raw);
+    }
+  }
+  // the value is (re)defined in the register class every later use names, so it is never copied back and forth
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) asm volatile("" : "+a"(qf[ks]));
 }
 
 template <bool kMask>
@@ -546,8 +634,8 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   // list: the workgroups that stream the same K / V run on the same XCD at the
   // same time and all but the first fetch of a tile hit in L2.
   int qtile, head, row, split;
+  const int nq = (a.q_tokens + kQTile - 1) / kQTile;
   {
-    const int nq = (a.q_tokens + kQTile - 1) / kQTile;
     const int total = nq * a.heads * a.rows * a.num_splits;
     const int xcd = blockIdx.x & 7;
     const int first = (int)(((int64_t)xcd * total) >> 3);
@@ -572,9 +660,15 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   tile_end = tile_end < ntiles ? tile_end : ntiles;
   const int n = tile_end - tile_begin;       // tiles this workgroup streams
 
-  const uint32_t lds_addr0 = (uint32_t)(uintptr_t)lds;
-  const char* kbase = reinterpret_cast<const char*>(a.k + row * a.k_st.row + head * a.k_st.head);
-  const char* vbase = reinterpret_cast<const char*>(a.v + row * a.v_st.row + head * a.v_st.head);
+  // (the transfers take their base addresses from scalar registers: say so to the compiler)
+  auto uniform = [](const void* ptr) {
+    const uint64_t x = reinterpret_cast<uint64_t>(ptr);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)x), hi = __builtin_amdgcn_readfirstlane((uint32_t)(x >> 32));
+    return reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
+  };
+  const uint32_t lds_addr0 = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)lds);
+  const char* kbase = uniform(a.k + row * a.k_st.row + head * a.k_st.head);
+  const char* vbase = uniform(a.v + row * a.v_st.row + head * a.v_st.head);
   const uint32_t k_tok_bytes = (uint32_t)(a.k_st.token * 2);
   const uint32_t v_tok_bytes = (uint32_t)(a.v_st.token * 2);
 
@@ -594,50 +688,62 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
     issue_matrix_tile(vbase, v_tok_bytes, v_ld, (tile_begin + T) * kKTile, seq, lds_addr0 + kLdsV(buf), wave_u, lane);
   };
 
+  // The transfers the first two slots need go out first; the query rows are
+  // fetched (and rotated) behind them, the rest of the look-ahead after that:
+  // ordinary loads return in order with the transfers, so whatever is issued
+  // ahead of the query rows is what the first wait for them also waits for.
   if (n > 0) {
-    // Every buffer starts with real (finite) data, also those whose tile does
-    // not exist: they are only ever met by all-zero weights.
     issue_k(0, 0);
     issue_v(0, 0);
     issue_k(n > 1 ? 1 : n - 1, 1);
-    issue_v(n > 1 ? 1 : n - 1, 1);
-    issue_k(n > 2 ? 2 : n - 1, 2);
-    issue_v(0, 2);              // stand-in for "V tile -1", met by the all-zero P(-1)
+    // V buffer 2 stands in for "V tile -1" in the first slot, where it meets the
+    // all-zero P(-1): any finite values do, so it is cleared (two 16-byte stores per lane)
+    {
+      const u32x4 zero = {0u, 0u, 0u, 0u};
+      *reinterpret_cast<__attribute__((address_space(3))) u32x4*>(lds + kLdsV(2) + tid * 16) = zero;
+      *reinterpret_cast<__attribute__((address_space(3))) u32x4*>(lds + kLdsV(2) + (kThreads + tid) * 16) = zero;
+    }
   }
 
-  // ---- this lane's query rows, as the B operand of S^T = K Q^T -------------
-  int q_row[kQB];
-  bf16x8 qf[kQB][8];
-#pragma unroll
-  for (int qb = 0; qb < kQB; ++qb) {
-    q_row[qb] = qtile * kQTile + wave * kQRowsPerWave + qb * 32 + (lane & 31);
-    const int q_row_c = q_row[qb] < a.q_tokens ? q_row[qb] : a.q_tokens - 1;
-    const uint16_t* qp = a.q + row * a.q_st.row + (int64_t)q_row_c * a.q_st.token + head * a.q_st.head + 8 * hf;
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      qf[qb][ks] = *reinterpret_cast<const bf16x8*>(qp + 16 * ks);
-      // with Q in AGPRs: the value is (re)defined in the register class every later
-      // use names, so it is never copied back and forth
-      if constexpr (kQB == 1) asm volatile("" : "+" SDV2_Q_REG(qf[qb][ks]));
-    }
+  // ---- this lane's query row -------------------------------------------------
+  const int q_row = qtile * kQTile + wave * kQBlock + (lane & 31);
+  bf16x8 qf[8];
+  {
+    const int q_row_c = q_row < a.q_tokens ? q_row : a.q_tokens - 1;
+    QueryRope rope;
+    rope.freqs = a.freqs;
+    rope.grid_w = a.grid_w; rope.frame_tokens = a.frame_tokens; rope.split_t = a.split_t; rope.split_h = a.split_h;
+    // (constant indices and selects: indexing the by-value argument block with a run-time
+    // row would move the whole block, its pointers included, out of scalar registers)
+    rope.start_frame = a.start_frame[0];
+    static_for<SDV2_MAX_ROWS - 1>([&](auto ic) {
+      constexpr int i = decltype(ic)::value + 1;
+      rope.start_frame = row == i ? a.start_frame[i] : rope.start_frame;
+    });
+    load_query(rope, a.q + row * a.q_st.row + (int64_t)q_row_c * a.q_st.token + head * a.q_st.head + 8 * hf, q_row_c,
+               hf, qf);
+  }
+  if (n > 0) {
+    // every buffer a slot may read starts with real (finite) data, also where the tile does not exist
+    issue_v(n > 1 ? 1 : n - 1, 1);
+    issue_k(n > 2 ? 2 : n - 1, 2);
   }
 
   // ---- per-lane LDS read addresses ------------------------------------------
   LaneConst c;
   c.c2 = a.scale_log2;
+  c.neg_ref = 0.f;
   c.hf = hf;
   if (kMask && a.mask_block_tokens > 0) {
     const int bt = a.mask_block_tokens;
     const int first = a.chunk_start[row];
     c.m_hi = __builtin_amdgcn_readfirstlane(first + a.q_tokens);
     c.wg_m_lo = __builtin_amdgcn_readfirstlane(first + ((qtile * kQTile) / bt + 1) * bt);
-#pragma unroll
-    for (int qb = 0; qb < kQB; ++qb) c.m_lo[qb] = first + (q_row[qb] / bt + 1) * bt;
+    c.m_lo = first + (q_row / bt + 1) * bt;
   } else {
     c.m_hi = 0;
     c.wg_m_lo = 0x7fffffff;
-#pragma unroll
-    for (int qb = 0; qb < kQB; ++qb) c.m_lo[qb] = 0x7fffffff;
+    c.m_lo = 0x7fffffff;
   }
   {
     // K (A operand): key = lane%32 of the block, chunk = 2*ks + hf
@@ -663,23 +769,19 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
       }
   }
 
-  f32x16 oacc[kQB][4];
+  f32x16 oacc[4];
 #pragma unroll
-  for (int qb = 0; qb < kQB; ++qb)
+  for (int db = 0; db < 4; ++db)
 #pragma unroll
-    for (int db = 0; db < 4; ++db)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) oacc[qb][db][i] = 0.f;
-  f32x16 s[2][kQB];
-  u32x4 p[2][kQB][2];
+    for (int i = 0; i < 16; ++i) oacc[db][i] = 0.f;
+  f32x16 s[2];
+  u32x4 p[2][2];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int qb = 0; qb < kQB; ++qb)
-#pragma unroll
-      for (int j = 0; j < 2; ++j) p[i][qb][j] = u32x4{0u, 0u, 0u, 0u};
-  float l_run[kQB] = {};             // this lane's share of each block's row sum
-  float m_run[kQB] = {};             // reference of the exponent: 0 in the fast pass
+    for (int j = 0; j < 2; ++j) p[i][j] = u32x4{0u, 0u, 0u, 0u};
+  float l_run = 0.f;                 // this lane's share of the row sum
+  float m_run = 0.f;                 // the row's exponent reference, in score units
   bool unsafe = false;
 
   // Tile T (64 keys) = blocks 2T, 2T+1, in K / V buffers T % 3.  Slot 2T needs
@@ -700,27 +802,12 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   // whatever finite data the buffers still hold.  In the first slot P(-1) is
   // zero likewise.
   const int key_end = seq < tile_end * kKTile ? seq : tile_end * kKTile;
-  // Checked once, after the last tile: a sum that overflowed stays inf or NaN, one
-  // that underflowed stays tiny.  With the mask inside the chunk a sum of exactly
-  // zero is legitimate when every key of this workgroup's range is hidden from
-  // the lane's query (its split then contributes nothing).
-  auto row_sums_unsafe = [&]() {
-    bool bad = false;
-#pragma unroll
-    for (int qb = 0; qb < kQB; ++qb) {
-      bool ok = l_run[qb] >= 0x1p-100f && l_run[qb] <= 0x1p100f;
-      if constexpr (kMask)
-        ok |= l_run[qb] == 0.f && tile_begin * kKTile >= c.m_lo[qb] && key_end <= c.m_hi;
-      bad |= !ok;
-    }
-    return __builtin_amdgcn_ballot_w64(bad) != 0;
-  };
   auto do_tile = [&](auto buf_c, int T) {
     constexpr int kB = decltype(buf_c)::value;              // T % 3
     constexpr int kBNext = (kB + 1) % kStages, kBPrev = (kB + 2) % kStages;
     const int key0 = (tile_begin + T) * kKTile;
     slot<kMask, 0, kLdsK(kB) + 32 * 256, kLdsVRel(kBPrev) + 32 * 256, true, true, true>(c, qf, s, p, oacc, l_run, key0,
-                                                                                key_end);
+                                                                                        key_end);
     if (T + 3 < n) {
       __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * kPieces));   // vmcnt: one K and one V tile's worth per wave
     } else {
@@ -735,10 +822,16 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   using B1 = std::integral_constant<int, 1>;
   using B2 = std::integral_constant<int, 2>;
 
-  const bool idle = __builtin_amdgcn_readfirstlane(qtile * kQTile + wave * kQRowsPerWave >= a.q_tokens);
+  const bool idle = __builtin_amdgcn_readfirstlane(qtile * kQTile + wave * kQBlock >= a.q_tokens);
   if (n > 0) {
-    __builtin_amdgcn_s_waitcnt(0x0F70);
-    __syncthreads();        // the first tiles and the Q fragments have arrived
+    // K tile 0 (and, for the first slot of the loop, V tile 0 and K tile 1) have
+    // landed once at most the last two transfers of an issuing wave are in flight
+    if (wave_u < kIssuers) {
+      __builtin_amdgcn_s_waitcnt(0x0070 | (2 * kPieces));   // vmcnt, and lgkmcnt(0) for the LDS clear
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0070);
+    }
+    __syncthreads();
     if (idle) {
       // No query row of this wave exists (the last query tile of a call is
       // rarely full).  The wave still moves its share of every K / V tile and
@@ -756,165 +849,234 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
         if (T + 2 < n) issue_v(T + 2, (T + 2) % kStages);
       }
     } else {
-    // S(0) alone fills the pipeline
-    slot<kMask, 1, kLdsK(0), 0, true, false, false>(c, qf, s, p, oacc, l_run, 0, key_end);
-    // Three tiles per trip, one per buffer; the last trip stops after the last
-    // real tile.  The skipped tiles sit behind uniform branches that no value
-    // is changed on, so the accumulators stay where they are on either way.
-    for (int T = 0; T < n; T += 3) {
-      do_tile(B0{}, T);
-      if (T + 1 < n) {
-        do_tile(B1{}, T + 1);
-        if (T + 2 < n) do_tile(B2{}, T + 2);
+      // S(0) alone fills the pipeline, and its largest score becomes the row's exponent reference
+      slot<kMask, 1, kLdsK(0), 0, true, false, false>(c, qf, s, p, oacc, l_run, 0, key_end);
+      mfma_drain<1>(oacc, s);
+      {
+        float ref = s[0][0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i) ref = vmax(ref, s[0][i]);
+        ref = half_max(ref);
+        ref = (ref > -0x1p120f && ref < 0x1p120f) ? ref : 0.f;      // also false for NaN
+        m_run = ref;
+        c.neg_ref = -ref * c.c2;
       }
-    }
-    // PV of the last block (odd -> p[1], second half of the last tile's V
-    // buffer) empties the pipeline.  The code addresses V buffer 2; the lane
-    // addresses are moved when the last tile sits in another buffer.
-    {
-      LaneConst cf = c;
-      const uint32_t shift = (uint32_t)(((n - 1) % kStages - 2) * kTileBytes);
+      // Three tiles per trip, one per buffer; the last trip stops after the last
+      // real tile.  The skipped tiles sit behind uniform branches that no value
+      // is changed on, so the accumulators stay where they are on either way.
+      for (int T = 0; T < n; T += 3) {
+        do_tile(B0{}, T);
+        if (T + 1 < n) {
+          do_tile(B1{}, T + 1);
+          if (T + 2 < n) do_tile(B2{}, T + 2);
+        }
+      }
+      // PV of the last block (odd -> p[1], second half of the last tile's V
+      // buffer) empties the pipeline.  The code addresses V buffer 2; the lane
+      // addresses are moved when the last tile sits in another buffer.
+      {
+        LaneConst cf = c;
+        const uint32_t shift = (uint32_t)(((n - 1) % kStages - 2) * kTileBytes);
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+        for (int db = 0; db < 4; ++db)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) cf.v_addr[db][j] = c.v_addr[db][j] + shift;
-      slot<kMask, 0, 0, kLdsVRel(2) + 32 * 256, false, true, false>(cf, qf, s, p, oacc, l_run, 0, key_end);
-    }
-    mfma_drain<0>(oacc, s);
-    unsafe = row_sums_unsafe();
+          for (int j = 0; j < 2; ++j) cf.v_addr[db][j] = c.v_addr[db][j] + shift;
+        slot<kMask, 0, 0, kLdsVRel(2) + 32 * 256, false, true, false>(cf, qf, s, p, oacc, l_run, 0, key_end);
+      }
+      mfma_drain<0>(oacc, s);
+      // Checked once, after the last tile: a sum that overflowed stays inf or NaN, one
+      // that underflowed stays tiny.  With the mask inside the chunk a sum of exactly
+      // zero is legitimate when every key of this workgroup's range is hidden from
+      // the lane's query (its split then contributes nothing).
+      {
+        const float l_tot = half_sum(l_run);
+        bool ok = l_tot >= 0x1p-100f && l_tot <= 0x1p100f;
+        if constexpr (kMask) ok |= l_tot == 0.f && tile_begin * kKTile >= c.m_lo && key_end <= c.m_hi;
+        unsafe = __builtin_amdgcn_ballot_w64(!ok) != 0;
+      }
     }
 
     // Did any wave of the workgroup see an unsafe row sum?  (LDS is free now.)
     __syncthreads();
-    if (tid == 0) *reinterpret_cast<__attribute__((address_space(3))) int*>(lds) = 0;
+    if (tid == 0) *reinterpret_cast<lds_int*>(lds) = 0;
     __syncthreads();
-    if (unsafe && lane == 0) *reinterpret_cast<__attribute__((address_space(3))) int*>(lds) = 1;
+    if (unsafe && lane == 0) *reinterpret_cast<lds_int*>(lds) = 1;
     __syncthreads();
-    const int redo = *reinterpret_cast<__attribute__((address_space(3))) int*>(lds);
+    const int redo = *reinterpret_cast<lds_int*>(lds);
     if (redo)
-      exact_pass(a, c, qf, oacc, m_run, l_run, kbase, vbase, k_tok_bytes, v_tok_bytes, k_ld, v_ld, tile_begin, n,
+      exact_pass(c, qf, oacc, m_run, l_run, unsafe, kbase, vbase, k_tok_bytes, v_tok_bytes, k_ld, v_ld, tile_begin, n,
                  seq, lds_addr0, lds, wave_u, lane);
   }
 
   // ---- epilogue ---------------------------------------------------------------
-  // A lane holds one query row's values scattered over the 128 dims, so direct
-  // stores would touch 32 rows with 16 or 32 bytes each.  Instead every wave
-  // stages one 32-row block at a time in its own 16 KB of the (now idle) LDS,
-  // 16-byte chunks XOR-swizzled by row, and writes whole rows of 256 bytes: bf16
-  // for the result of an unsplit call, scaled fp16 for the partial result of a
-  // split call (plus its scale and log-sum-exp).  LDS operations of
-  // one wave complete in order, so the block needs no barrier of its own.
   __syncthreads();                    // every wave is done with the K / V buffers
-  lds_char* stage = lds + wave * kStageBytes;
-  const int q0 = qtile * kQTile + wave * kQRowsPerWave;
-  if (idle) return;
-#pragma unroll
-  for (int qb = 0; qb < kQB; ++qb) {
-    const float l_tot = half_sum(l_run[qb]);
-    const float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
-    const int r = lane & 31;
-    if (a.num_splits == 1) {
-#pragma unroll
-      for (int db = 0; db < 4; ++db)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          u32x2 w;
-          w[0] = pack_bf16x2(oacc[qb][db][4 * g] * inv, oacc[qb][db][4 * g + 1] * inv);
-          w[1] = pack_bf16x2(oacc[qb][db][4 * g + 2] * inv, oacc[qb][db][4 * g + 3] * inv);
-          const int chunk = db * 4 + g;
-          *reinterpret_cast<__attribute__((address_space(3))) u32x2*>(
-              stage + r * 256 + ((chunk ^ (r & 15)) << 4) + hf * 8) = w;
-        }
-      uint16_t* dst = a.out + row * a.o_st.row + head * a.o_st.head + (int64_t)(q0 + qb * 32) * a.o_st.token;
-      const int j = lane & 15;
-#pragma unroll
-      for (int it = 0; it < 8; ++it) {
-        const int rr = 4 * it + (lane >> 4);
-        const u32x4 w = *reinterpret_cast<__attribute__((address_space(3))) const u32x4*>(
-            stage + rr * 256 + ((j ^ (rr & 15)) << 4));
-        if (q0 + qb * 32 + rr < a.q_tokens) *reinterpret_cast<u32x4*>(dst + rr * a.o_st.token + j * 8) = w;
-      }
-    } else {
-      // Partial result of a key range: the normalised row divided by its largest
-      // magnitude, as fp16 (values in [-1, 1]: 11 bits against the row's scale,
-      // sixteen times finer than the bf16 of the final result), plus that scale
-      // and the log-sum-exp.  Half the bytes of an fp32 partial, written and read.
+  const int block = qtile * kWaves + wave;              // this wave's 32-row block within the (row, head)
+  float l_tot = half_sum(l_run);
+  float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
+
+  if (a.num_splits > 1) {
+    // Partial result of a key range: the normalised row divided by its largest
+    // magnitude, as fp16 (values in [-1, 1]: 11 bits against the row's scale,
+    // sixteen times finer than the bf16 of the final result), plus that scale
+    // and the log-sum-exp.  Stored in register order - 16-byte piece j of a lane
+    // holds its accumulator registers 8 j .. 8 j + 7 - so that every store and,
+    // later, every load of the combining workgroup is one contiguous kilobyte
+    // per wave and the values come back to the registers they left.
+    const int64_t slab = (int64_t)a.rows * a.heads * a.q_blocks;
+    const int64_t blk0 = ((int64_t)row * a.heads + head) * a.q_blocks + block;
+    if (!idle) {
       float amax = 0.f;
 #pragma unroll
       for (int db = 0; db < 4; ++db)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) amax = vmax(amax, __builtin_fabsf(oacc[qb][db][i]));
+        for (int i = 0; i < 16; ++i) amax = vmax(amax, __builtin_fabsf(oacc[db][i]));
       amax = half_max(amax) * inv;
       const float row_scale = amax > 0.f && amax < INFINITY ? amax : 1.0f;
       const float to_unit = inv / row_scale;
+      const int64_t blk = split * slab + blk0;
+      // piece j of the lane (its accumulator registers 8 j .. 8 j + 7 as fp16) lies j KB into the block
+      char* dst = reinterpret_cast<char*>(a.part_o + blk * kPartBlockHalves + lane * 8);
 #pragma unroll
-      for (int db = 0; db < 4; ++db)
+      for (int half = 0; half < 2; ++half) {
+        u32x4 w[4];
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          u32x2 w;
-          w[0] = pack_f16x2(oacc[qb][db][4 * g] * to_unit, oacc[qb][db][4 * g + 1] * to_unit);
-          w[1] = pack_f16x2(oacc[qb][db][4 * g + 2] * to_unit, oacc[qb][db][4 * g + 3] * to_unit);
-          const int chunk = db * 4 + g;
-          *reinterpret_cast<__attribute__((address_space(3))) u32x2*>(
-              stage + r * 256 + ((chunk ^ (r & 15)) << 4) + hf * 8) = w;
+        for (int jj = 0; jj < 4; ++jj) {
+          const int j = 4 * half + jj, db = j >> 1, i0 = 8 * (j & 1);
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            w[jj][e] = pack_f16x2(oacc[db][i0 + 2 * e] * to_unit, oacc[db][i0 + 2 * e + 1] * to_unit);
         }
-      const int64_t prow0 = (((int64_t)split * a.rows + row) * a.heads + head) * a.q_tokens + q0 + qb * 32;
-      if (hf == 0 && q_row[qb] < a.q_tokens) {
-        a.part_lse[prow0 + r] = l_tot > 0.f ? m_run[qb] * c.c2 + __builtin_amdgcn_logf(l_tot) : -INFINITY;
-        a.part_scale[prow0 + r] = row_scale;
+        store_coherent_x4(dst + half * 4096, w[0], w[1], w[2], w[3]);
       }
-      uint16_t* dst = a.part_o + prow0 * kD;
-      const int j = lane & 15;
-#pragma unroll
-      for (int it = 0; it < 8; ++it) {
-        const int rr = 4 * it + (lane >> 4);
-        const u32x4 w = *reinterpret_cast<__attribute__((address_space(3))) const u32x4*>(
-            stage + rr * 256 + ((j ^ (rr & 15)) << 4));
-        if (q0 + qb * 32 + rr < a.q_tokens) *reinterpret_cast<u32x4*>(dst + rr * kD + j * 8) = w;
+      if (hf == 0) {
+        store_coherent(a.part_lse + blk * kQBlock + lane,
+                       l_tot > 0.f ? m_run * c.c2 + __builtin_amdgcn_logf(l_tot) : -INFINITY);
+        store_coherent(a.part_scale + blk * kQBlock + lane, row_scale);
       }
     }
-  }
-}
+    // Ticket.  Every wave has waited for its stores to be acknowledged before the
+    // barrier; then one lane draws.  The workgroup that draws the last ticket of
+    // its (row, head, query tile) finds every other range's results in memory,
+    // and leaves the ticket at zero for the next call.
+    __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0)
+    __syncthreads();
+    if (tid == 0) {
+      int32_t* ticket = a.tickets + ((int64_t)row * a.heads + head) * nq + qtile;
+      const int drawn = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const int last = drawn == a.num_splits - 1;
+      if (last) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      *reinterpret_cast<lds_int*>(lds) = last;
+    }
+    __syncthreads();
+    if (*reinterpret_cast<lds_int*>(lds) == 0 || idle) return;
+    __syncthreads();                  // (the flag word lies in wave 0's staging area)
 
-// Combine the per-split partial results: out = sum_s 2^(lse_s - LSE) O_s.
-// One 16-lane group per (row, head, query); each lane owns 8 of the 128 dims.
-__global__ __launch_bounds__(256)
-void swa_attn_merge_kernel(const AttnKernelArgs a) {
-  const int64_t nq = (int64_t)a.rows * a.heads * a.q_tokens;
-  const int64_t idx = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
-  if (idx >= nq) return;
-  const int lane = threadIdx.x & 15;
-  const int q_row = (int)(idx % a.q_tokens);
-  const int head = (int)((idx / a.q_tokens) % a.heads);
-  const int row = (int)(idx / ((int64_t)a.q_tokens * a.heads));
-
-  float lse_max = -INFINITY;
-  for (int s = 0; s < a.num_splits; ++s) lse_max = fmaxf(lse_max, a.part_lse[s * nq + idx]);
-  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  float wsum = 0.f;
-  for (int s = 0; s < a.num_splits; ++s) {
-    const float lse = a.part_lse[s * nq + idx];
-    const float w = lse == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(lse - lse_max);
-    wsum += w;
-    const float ws = w * a.part_scale[s * nq + idx];          // weight times the row's fp16 scale
-    const f16x8 x = *reinterpret_cast<const f16x8*>(a.part_o + (s * nq + idx) * kD + lane * 8);
+    // combine: out = sum_s 2^(lse_s - LSE) O_s over the ranges in their fixed
+    // order (every range, this workgroup's own included, as it lies in memory:
+    // the sum does not depend on which workgroup happens to be last)
+    const int r32 = lane & 31;
+    constexpr int kBatch = 8;         // ranges whose statistics are fetched together
+    float wsum = 0.f;
+    float lse[kBatch], scale[kBatch], ws[kBatch];
+    // log-sum-exp and row scale of the ranges of a batch; the loads go out together
+    auto fetch = [&](int s0) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) acc[i] += ws * static_cast<float>(x[i]);
+      for (int u = 0; u < kBatch; ++u) {
+        const int sp = s0 + u < a.num_splits ? s0 + u : a.num_splits - 1;
+        lse[u] = load_coherent(a.part_lse + (sp * slab + blk0) * kQBlock + r32);
+        scale[u] = load_coherent(a.part_scale + (sp * slab + blk0) * kQBlock + r32);
+      }
+    };
+    fetch(0);
+    float lse_max = lse[0];
+#pragma unroll
+    for (int u = 1; u < kBatch; ++u) lse_max = fmaxf(lse_max, lse[u]);         // (entries past the last range repeat it)
+    for (int sp = kBatch; sp < a.num_splits; ++sp)
+      lse_max = fmaxf(lse_max, load_coherent(a.part_lse + (sp * slab + blk0) * kQBlock + r32));
+#pragma unroll
+    for (int db = 0; db < 4; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) oacc[db][i] = 0.f;
+    for (int s0 = 0; s0 < a.num_splits; s0 += kBatch) {
+      if (s0 > 0) fetch(s0);
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        const float w = (s0 + u >= a.num_splits || lse[u] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(lse[u] - lse_max);
+        wsum += w;
+        ws[u] = w * scale[u];         // weight times the row's fp16 scale
+      }
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) {
+        if (s0 + u >= a.num_splits) break;
+        u32x4 x[8];
+        load_coherent_x8(
+            reinterpret_cast<const char*>(a.part_o + ((s0 + u) * slab + blk0) * kPartBlockHalves + lane * 8), x);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int db = j >> 1, i0 = 8 * (j & 1);
+          const f16x8 h = __builtin_bit_cast(f16x8, x[j]);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) oacc[db][i0 + e] += ws[u] * static_cast<float>(h[e]);
+        }
+      }
+    }
+    inv = wsum > 0.f ? 1.0f / wsum : 0.f;
+  } else if (idle) {
+    return;
   }
-  const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
-  uint4 o;
-  o.x = pack_bf16x2(acc[0] * inv, acc[1] * inv);
-  o.y = pack_bf16x2(acc[2] * inv, acc[3] * inv);
-  o.z = pack_bf16x2(acc[4] * inv, acc[5] * inv);
-  o.w = pack_bf16x2(acc[6] * inv, acc[7] * inv);
-  uint16_t* op = a.out + row * a.o_st.row + (int64_t)q_row * a.o_st.token + head * a.o_st.head + lane * 8;
-  *reinterpret_cast<uint4*>(op) = o;
+
+  // A lane holds one query row's values scattered over the 128 dims, so direct
+  // stores would touch 32 rows with 16 or 32 bytes each.  Instead every wave
+  // stages its 32-row block in its own 16 KB of the (now idle) LDS, 16-byte
+  // chunks XOR-swizzled by row, and writes whole rows of 256 bytes.  LDS
+  // operations of one wave complete in order, so the block needs no barrier of
+  // its own.
+  lds_char* stage = lds + wave * kStageBytes;
+  const int q0 = qtile * kQTile + wave * kQBlock;
+  const int r = lane & 31;
+#pragma unroll
+  for (int db = 0; db < 4; ++db)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      u32x2 w;
+      w[0] = pack_bf16x2(oacc[db][4 * g] * inv, oacc[db][4 * g + 1] * inv);
+      w[1] = pack_bf16x2(oacc[db][4 * g + 2] * inv, oacc[db][4 * g + 3] * inv);
+      const int chunk = db * 4 + g;
+      *reinterpret_cast<__attribute__((address_space(3))) u32x2*>(stage + r * 256 + ((chunk ^ (r & 15)) << 4) + hf * 8) =
+          w;
+    }
+  uint16_t* dst = a.out + row * a.o_st.row + head * a.o_st.head + (int64_t)q0 * a.o_st.token;
+  const int j = lane & 15;
+#pragma unroll
+  for (int it = 0; it < 8; ++it) {
+    const int rr = 4 * it + (lane >> 4);
+    const u32x4 w = *reinterpret_cast<__attribute__((address_space(3))) const u32x4*>(
+        stage + rr * 256 + ((j ^ (rr & 15)) << 4));
+    if (q0 + rr < a.q_tokens) *reinterpret_cast<u32x4*>(dst + rr * a.o_st.token + j * 8) = w;
+  }
 }
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 bool stride_ok(const sdv2_stride3& s) { return s.row % 8 == 0 && s.token % 8 == 0 && s.head % 8 == 0; }
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// layout of the split-KV workspace: tickets, partial outputs, log-sum-exps, row scales
+struct WorkspaceLayout {
+  size_t tickets, part_o, part_lse, part_scale, total;
+};
+WorkspaceLayout workspace_layout(int32_t rows, int32_t q_tokens, int32_t heads, int32_t num_splits) {
+  const size_t nq = (size_t)(q_tokens + kQTile - 1) / kQTile;
+  const size_t blocks = (size_t)rows * heads * ((q_tokens + kQBlock - 1) / kQBlock);
+  WorkspaceLayout w;
+  (void)nq;
+  w.tickets = 0;
+  w.part_o = (size_t)kMaxTickets * sizeof(int32_t);
+  w.part_lse = w.part_o + (size_t)num_splits * blocks * kPartBlockHalves * sizeof(uint16_t);
+  w.part_scale = w.part_lse + align_up((size_t)num_splits * blocks * kQBlock * sizeof(float), 256);
+  w.total = w.part_scale + align_up((size_t)num_splits * blocks * kQBlock * sizeof(float), 256);
+  return w;
+}
 
 }  // namespace
 
@@ -955,10 +1117,11 @@ extern "C" int sdv2_swa_attn_default_splits(int32_t rows, int32_t q_tokens, int3
   // One workgroup per CU.  With s key-range splits there are qwork * s
   // workgroups; they run in ceil(qwork * s / 256) rounds, each as long as one
   // workgroup's tile count plus a fixed start / end cost of about three tile
-  // times.  Writing and merging the partial results
+  // times.  Writing and combining the partial results
   // costs roughly one tile time per 3.5 MB of them per split.  Constants fitted
   // to measurements on the five benchmark shapes.
   const int64_t qwork = (int64_t)rows * heads * ((q_tokens + kQTile - 1) / kQTile);
+  if (qwork > kMaxTickets) return 1;
   const int ntiles = (max_seq_len + kKTile - 1) / kKTile;
   const double partial_tiles = (double)rows * heads * q_tokens * kD * 4 / 7.0e6;
   int best = 1;
@@ -976,10 +1139,8 @@ extern "C" int sdv2_swa_attn_default_splits(int32_t rows, int32_t q_tokens, int3
 extern "C" size_t sdv2_swa_attn_workspace_bytes(int32_t rows, int32_t q_tokens, int32_t heads,
                                                  int32_t max_seq_len, int32_t num_splits) {
   if (num_splits <= 0) num_splits = sdv2_swa_attn_default_splits(rows, q_tokens, heads, max_seq_len);
-  if (num_splits <= 1) return 0;
-  const size_t nq = (size_t)rows * heads * q_tokens;
-  return align_up((size_t)num_splits * nq * kD * sizeof(uint16_t), 256) +
-         2 * align_up((size_t)num_splits * nq * sizeof(float), 256);
+  if (num_splits <= 1 || rows <= 0 || q_tokens <= 0 || heads <= 0) return 0;
+  return workspace_layout(rows, q_tokens, heads, num_splits).total;
 }
 
 extern "C" int sdv2_swa_attn_fwd(const sdv2_attn_params* p) {
@@ -1018,9 +1179,10 @@ int attn_fwd(const sdv2_attn_params* p, void* workspace, size_t workspace_bytes)
   int splits = p->num_splits > 0 ? p->num_splits
                                  : sdv2_swa_attn_default_splits(p->rows, p->q_tokens, p->heads, p->max_seq_len);
   if (splits > 64) return SDV2_ERR_INVALID_ARG;
-  // measurement hook: a split call can be told to run only one of its two kernels
-  const int stages = splits > 1 ? sdv2::attention_stages() : SDV2_STAGE_ALL;
   if ((int64_t)p->rows * splits > 65535) return SDV2_ERR_INVALID_ARG;
+  // more (row, head, query tile) groups than there are ticket words: such a grid fills the chip unsplit
+  if (splits > 1 && (int64_t)p->rows * p->heads * ((p->q_tokens + kQTile - 1) / kQTile) > kMaxTickets)
+    return SDV2_ERR_UNSUPPORTED;
 
   AttnKernelArgs a{};
   a.q = static_cast<const uint16_t*>(p->q);
@@ -1041,50 +1203,64 @@ int attn_fwd(const sdv2_attn_params* p, void* workspace, size_t workspace_bytes)
     a.mask_block_tokens = p->mask_block_tokens;
   }
 
+  if (p->rope_freqs) {
+    // q arrives before RoPE and is rotated as it is loaded; the chunk is grid_f whole frames of grid_h x grid_w
+    if (p->rows > SDV2_MAX_ROWS || !p->rope_start_frame) return SDV2_ERR_INVALID_ARG;
+    if (p->rope_grid_h <= 0 || p->rope_grid_w <= 0) return SDV2_ERR_INVALID_ARG;
+    const int64_t frame_tokens = (int64_t)p->rope_grid_h * p->rope_grid_w;
+    if (p->q_tokens % frame_tokens != 0) return SDV2_ERR_INVALID_ARG;
+    const int64_t grid_f = p->q_tokens / frame_tokens;
+    if (p->rope_grid_h > p->rope_freq_rows || p->rope_grid_w > p->rope_freq_rows) return SDV2_ERR_OUT_OF_RANGE;
+    for (int i = 0; i < p->rows; ++i) {
+      if (p->rope_start_frame[i] < 0 || p->rope_start_frame[i] + grid_f > p->rope_freq_rows)
+        return SDV2_ERR_OUT_OF_RANGE;
+      a.start_frame[i] = p->rope_start_frame[i];
+    }
+    a.freqs = reinterpret_cast<const double2*>(p->rope_freqs);
+    a.grid_w = p->rope_grid_w;
+    a.frame_tokens = (int32_t)frame_tokens;
+    // column split of the table: c - 2*(c/3) | c/3 | c/3  (causal_model.py:77-78)
+    const int third = (kD / 2) / 3;
+    a.split_t = kD / 2 - 2 * third;
+    a.split_h = a.split_t + third;
+  }
+
+  a.q_blocks = (p->q_tokens + kQBlock - 1) / kQBlock;
   if (splits > 1) {
-    const size_t need = sdv2_swa_attn_workspace_bytes(p->rows, p->q_tokens, p->heads, p->max_seq_len, splits);
-    if (!workspace || workspace_bytes < need) return SDV2_ERR_WORKSPACE;
+    const WorkspaceLayout w = workspace_layout(p->rows, p->q_tokens, p->heads, splits);
+    if (!workspace || workspace_bytes < w.total) return SDV2_ERR_WORKSPACE;
     if (reinterpret_cast<uintptr_t>(workspace) & 255) return SDV2_ERR_INVALID_ARG;
-    const size_t nq = (size_t)p->rows * p->heads * p->q_tokens;
     char* ws = static_cast<char*>(workspace);
-    a.part_o = reinterpret_cast<uint16_t*>(ws);
-    ws += align_up((size_t)splits * nq * kD * sizeof(uint16_t), 256);
-    a.part_lse = reinterpret_cast<float*>(ws);
-    a.part_scale = reinterpret_cast<float*>(ws + align_up((size_t)splits * nq * sizeof(float), 256));
+    a.tickets = reinterpret_cast<int32_t*>(ws + w.tickets);
+    a.part_o = reinterpret_cast<uint16_t*>(ws + w.part_o);
+    a.part_lse = reinterpret_cast<float*>(ws + w.part_lse);
+    a.part_scale = reinterpret_cast<float*>(ws + w.part_scale);
   }
 
   hipStream_t stream = static_cast<hipStream_t>(p->stream);
   const int64_t items = (int64_t)((p->q_tokens + kQTile - 1) / kQTile) * p->heads * p->rows * splits;
   if (items > (1 << 28)) return SDV2_ERR_INVALID_ARG;
   dim3 grid((unsigned)(8 * ((items + 7) / 8)));
-  if (stages != SDV2_STAGE_MERGE) {
-    // The tile buffers (96 KB) or the epilogue staging (16 KB per wave) exceed the static limit:
-    // ask for the dynamic size once per device.
-    // The kernel exists twice: the mask inside the chunk costs the plain
-    // variant about 2 % even when it is off, so it gets its own code.
-    static std::atomic<bool> lds_ready[kMaxDevices];
-    int device = 0;
-    if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return SDV2_ERR_LAUNCH;
-    if (!lds_ready[device].load(std::memory_order_acquire)) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(swa_attn_fwd_kernel<false>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess ||
-          hipFuncSetAttribute(reinterpret_cast<const void*>(swa_attn_fwd_kernel<true>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess)
-        return SDV2_ERR_LAUNCH;
-      lds_ready[device].store(true, std::memory_order_release);
-    }
-    if (a.mask_block_tokens > 0)
-      sdv2::launch_timed(SDV2_KERNEL_ATTENTION, swa_attn_fwd_kernel<true>, grid, dim3(kThreads), kLdsBytes, stream, a);
-    else
-      sdv2::launch_timed(SDV2_KERNEL_ATTENTION, swa_attn_fwd_kernel<false>, grid, dim3(kThreads), kLdsBytes, stream, a);
-    if (hipGetLastError() != hipSuccess) return SDV2_ERR_LAUNCH;
+  // The tile buffers (96 KB) or the epilogue staging (16 KB per wave) exceed the static limit:
+  // ask for the dynamic size once per device.
+  // The kernel exists twice: the mask inside the chunk costs the plain
+  // variant about 2 % even when it is off, so it gets its own code.
+  static std::atomic<bool> lds_ready[kMaxDevices];
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return SDV2_ERR_LAUNCH;
+  if (!lds_ready[device].load(std::memory_order_acquire)) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(swa_attn_fwd_kernel<false>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess ||
+        hipFuncSetAttribute(reinterpret_cast<const void*>(swa_attn_fwd_kernel<true>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes) != hipSuccess)
+      return SDV2_ERR_LAUNCH;
+    lds_ready[device].store(true, std::memory_order_release);
   }
-  if (splits > 1 && stages != SDV2_STAGE_PARTIAL) {
-    const int64_t nq = (int64_t)p->rows * p->heads * p->q_tokens;
-    sdv2::launch_timed(SDV2_KERNEL_MERGE, swa_attn_merge_kernel, dim3((unsigned)((nq + 15) / 16)), dim3(256), 0, stream,
-                       a);
-    if (hipGetLastError() != hipSuccess) return SDV2_ERR_LAUNCH;
-  }
+  if (a.mask_block_tokens > 0)
+    sdv2::launch_timed(SDV2_KERNEL_ATTENTION, swa_attn_fwd_kernel<true>, grid, dim3(kThreads), kLdsBytes, stream, a);
+  else
+    sdv2::launch_timed(SDV2_KERNEL_ATTENTION, swa_attn_fwd_kernel<false>, grid, dim3(kThreads), kLdsBytes, stream, a);
+  if (hipGetLastError() != hipSuccess) return SDV2_ERR_LAUNCH;
   return SDV2_OK;
 }
 

@@ -259,12 +259,18 @@ def causal_rope_apply(x: torch.Tensor, grid_sizes, freqs: torch.Tensor, start_fr
 _WORKSPACES: dict = {}
 
 
+def new_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
+    """A split-KV workspace as the library wants it: zero-filled once (its
+    ticket words start at zero and every call leaves them there)."""
+    return torch.zeros(max(nbytes, 1), dtype=torch.uint8, device=dev)
+
+
 def _workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
     """Per-device scratch for split-KV partials, grown on demand and reused
-    (stream-ordered reuse is safe: merge always follows its split kernel)."""
+    (safe for stream-ordered use on one stream: a call is one launch)."""
     ws = _WORKSPACES.get(dev)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=dev)
+        ws = new_workspace(dev, nbytes)
         _WORKSPACES[dev] = ws
     return ws
 
@@ -296,8 +302,14 @@ def swa_attention(
     chunk_key_start: Optional[torch.Tensor] = None,
     mask_block_tokens: int = 0,
     static_scratch: bool = False,
+    rope: Optional[Tuple[torch.Tensor, Sequence[int], Sequence[int]]] = None,
 ) -> torch.Tensor:
     """out[b] = softmax(q[b] k_cache[b,:seq_lens[b]]^T * scale) v_cache[b,:seq_lens[b]].
+
+    ``rope`` = (:func:`device_freqs` table, (grid_h, grid_w), start frame per
+    row): q is the query BEFORE RoPE and is rotated inside the kernel exactly as
+    :func:`kv_append_rope` would have rotated it (S must be whole frames).  A
+    caller-owned ``workspace`` must come from :func:`new_workspace` (zero-filled).
 
     ``static_scratch`` takes the library's allocation-free entry point
     (``sdv2_swa_attn_fwd_static``): partial results of a split call go to device
@@ -351,6 +363,16 @@ def swa_attention(
         chunk_key_start = chunk_starts_tensor(chunk_key_start, rows, q_tokens, max_seq_len, dev)
         p.mask_block_tokens = int(mask_block_tokens)
         p.chunk_key_start = chunk_key_start.data_ptr()
+    if rope is not None:
+        table, grid_hw, start_frames = rope
+        if table.dtype != torch.float64 or not table.is_contiguous() or table.device != dev:
+            raise RuntimeError("rope table must be the contiguous float64 view from device_freqs() on q's device")
+        if len(start_frames) != rows:
+            raise RuntimeError("rope needs one start frame per row")
+        frames = _i64_array(start_frames)
+        p.rope_freqs, p.rope_freq_rows = table.data_ptr(), table.shape[0]
+        p.rope_grid_h, p.rope_grid_w = int(grid_hw[0]), int(grid_hw[1])
+        p.rope_start_frame = C.cast(frames, C.POINTER(C.c_int64))
     with torch.cuda.device(dev):
         if static_scratch:
             _capi.check(lib.sdv2_swa_attn_fwd_static(C.byref(p)), "sdv2_swa_attn_fwd_static")
@@ -497,7 +519,7 @@ class LayerLauncher:
         return (tuple(t.shape), tuple(t.stride()), t.dtype)
 
     def __init__(self, k_cache, v_cache, global_end_index, local_end_index, freqs_table, grid, q_like, k_like=None,
-                 v_like=None, qk_norm=None):
+                 v_like=None, qk_norm=None, rope_in_attention=True):
         k_like = q_like if k_like is None else k_like
         v_like = q_like if v_like is None else v_like
         rows, tokens, heads, _ = q_like.shape
@@ -515,17 +537,24 @@ class LayerLauncher:
                           tuple(v_cache.stride()), global_end_index.data_ptr(), local_end_index.data_ptr())
         self.k_cache, self.v_cache = k_cache, v_cache
         self.lib = _capi.lib()
-        self.roped_q = torch.empty((rows, tokens, heads, HEAD_DIM), dtype=torch.bfloat16, device=dev)
+        # The query is rotated where it is consumed, inside the attention kernel,
+        # so the append moves K and V only.  With the q / k norm folded into the
+        # append (which needs whole tokens of q) or on request, the append rotates
+        # q as well and hands the attention the rotated copy in ``roped_q``.
+        self.rope_in_attention = bool(rope_in_attention) and qk_norm is None
+        self.roped_q = None if self.rope_in_attention else torch.empty(
+            (rows, tokens, heads, HEAD_DIM), dtype=torch.bfloat16, device=dev)
         self.sf = (C.c_int64 * rows)()
         self.ds = (C.c_int64 * rows)()
         self.ng = (C.c_int64 * rows)()
         self.nl = (C.c_int64 * rows)()
 
         ap = _capi.AppendParams()
-        ap.q_in_stride = _stride3(q_like, "q")
         ap.k_in_stride = _stride3(k_like, "k")
         ap.v_in_stride = _stride3(v_like, "v")
-        ap.q_out, ap.q_out_stride = self.roped_q.data_ptr(), _stride3(self.roped_q, "q_out")
+        if not self.rope_in_attention:
+            ap.q_in_stride = _stride3(q_like, "q")
+            ap.q_out, ap.q_out_stride = self.roped_q.data_ptr(), _stride3(self.roped_q, "q_out")
         ap.k_cache, ap.k_cache_stride = k_cache.data_ptr(), _stride3(k_cache, "k_cache")
         ap.v_cache, ap.v_cache_stride = v_cache.data_ptr(), _stride3(v_cache, "v_cache")
         ap.freqs, ap.freq_rows = freqs_table.data_ptr(), freqs_table.shape[0]
@@ -548,7 +577,13 @@ class LayerLauncher:
         self.freqs_table = freqs_table
 
         at = _capi.AttnParams()
-        at.q, at.q_stride = self.roped_q.data_ptr(), _stride3(self.roped_q, "q")
+        if self.rope_in_attention:
+            at.q_stride = _stride3(q_like, "q")
+            at.rope_freqs, at.rope_freq_rows = freqs_table.data_ptr(), freqs_table.shape[0]
+            at.rope_grid_h, at.rope_grid_w = int(grid[1]), int(grid[2])
+            at.rope_start_frame = C.cast(self.sf, C.POINTER(C.c_int64))
+        else:
+            at.q, at.q_stride = self.roped_q.data_ptr(), _stride3(self.roped_q, "q")
         at.k_cache, at.k_stride = k_cache.data_ptr(), _stride3(k_cache, "k_cache")
         at.v_cache, at.v_stride = v_cache.data_ptr(), _stride3(v_cache, "v_cache")
         at.rows, at.q_tokens, at.heads, at.head_dim = rows, tokens, heads, HEAD_DIM
@@ -556,7 +591,7 @@ class LayerLauncher:
         self.span = -1
         self.out_stride = None
         self.forced_splits = 0                       # 0 = the library's own choice
-        self.timers = (None, None, None)
+        self.timers = (None, None)
 
     def matches(self, q, k, v, kv_cache, freqs_table, qk_norm=None) -> bool:
         if (self._sig(q), self._sig(k), self._sig(v)) != self.in_sig or freqs_table is not self.freqs_table:
@@ -588,7 +623,11 @@ class LayerLauncher:
             self.ds[i] = plan.dst_start[i]
             self.ng[i] = plan.new_global_end[i]
             self.nl[i] = plan.new_local_end[i]
-        ap.q_in, ap.k_in, ap.v_in = q.data_ptr(), k.data_ptr(), v.data_ptr()
+        ap.k_in, ap.v_in = k.data_ptr(), v.data_ptr()
+        if self.rope_in_attention:
+            at.q = q.data_ptr()
+        else:
+            ap.q_in = q.data_ptr()
         stream = _stream_ptr(self.dev)
         ap.stream = stream
         span = plan.max_seq_len
@@ -613,35 +652,24 @@ class LayerLauncher:
         at.stream = stream
         return out
 
-    def set_timers(self, append: Optional[KernelTimer] = None, attention: Optional[KernelTimer] = None,
-                   merge: Optional[KernelTimer] = None) -> None:
+    def set_timers(self, append: Optional[KernelTimer] = None, attention: Optional[KernelTimer] = None) -> None:
         """Attach (or, with None, detach) kernel timers for the next launches."""
-        self.timers = (append, attention, merge)
+        self.timers = (append, attention)
 
     def run_append(self) -> None:
         if self.timers[0] is not None:
             self.timers[0].arm(_capi.KERNEL_APPEND)
         _capi.check(self.lib.sdv2_kv_append_rope(self.ap_ref), "sdv2_kv_append_rope")
 
-    def run_attention(self, stages: int = _capi.STAGE_ALL) -> None:
-        """``stages`` other than STAGE_ALL runs one kernel of a split call only
-        (measurement hook; restored before returning)."""
-        if self.timers[1] is not None and stages != _capi.STAGE_MERGE:
+    def run_attention(self) -> None:
+        if self.timers[1] is not None:
             self.timers[1].arm(_capi.KERNEL_ATTENTION)
-        if self.timers[2] is not None and stages != _capi.STAGE_PARTIAL and self.at.num_splits > 1:
-            self.timers[2].arm(_capi.KERNEL_MERGE)
-        if stages != _capi.STAGE_ALL:
-            _capi.check(self.lib.sdv2_profile_attention_stages(stages), "sdv2_profile_attention_stages")
-        try:
-            _capi.check(self.lib.sdv2_swa_attn_fwd(self.at_ref), "sdv2_swa_attn_fwd")
-        finally:
-            if stages != _capi.STAGE_ALL:
-                self.lib.sdv2_profile_attention_stages(_capi.STAGE_ALL)
+        _capi.check(self.lib.sdv2_swa_attn_fwd(self.at_ref), "sdv2_swa_attn_fwd")
 
     def launch(self, q, k, v, start_frames, plan, seq_lens: Optional[torch.Tensor] = None,
                mask_block_tokens: int = 0, dst_start_override: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Append + attention for one call; returns the attention output
-        [rows, S, H, 128].  The roped query stays in ``self.roped_q``."""
+        [rows, S, H, 128]."""
         out = self.patch(q, k, v, start_frames, plan, seq_lens, mask_block_tokens, dst_start_override)
         if _current_device_index() != self.dev.index:
             with torch.cuda.device(self.dev):

@@ -70,8 +70,8 @@ int main(void) {
   /* struct layouts, for the bindings to compare themselves with */
   printf("layout sdv2_append_params size=%zu stream=%zu dst_start_override=%zu\n", sizeof(sdv2_append_params),
          offsetof(sdv2_append_params, stream), offsetof(sdv2_append_params, dst_start_override));
-  printf("layout sdv2_attn_params size=%zu stream=%zu chunk_key_start=%zu\n", sizeof(sdv2_attn_params),
-         offsetof(sdv2_attn_params, stream), offsetof(sdv2_attn_params, chunk_key_start));
+  printf("layout sdv2_attn_params size=%zu stream=%zu rope_start_frame=%zu\n", sizeof(sdv2_attn_params),
+         offsetof(sdv2_attn_params, stream), offsetof(sdv2_attn_params, rope_start_frame));
   printf("layout sdv2_sink_sim_params size=%zu stream=%zu override_rows=%zu\n", sizeof(sdv2_sink_sim_params),
          offsetof(sdv2_sink_sim_params, stream), offsetof(sdv2_sink_sim_params, override_rows));
   printf("layout sdv2_relayout_params size=%zu stream=%zu global_end_shift=%zu\n", sizeof(sdv2_relayout_params),
@@ -86,8 +86,6 @@ int main(void) {
   expect("time_next(unknown kernel)", sdv2_profile_time_next(SDV2_KERNEL_COUNT, NULL, NULL), SDV2_ERR_INVALID_ARG);
   expect("time_next(start only)", sdv2_profile_time_next(SDV2_KERNEL_APPEND, &failures, NULL), SDV2_ERR_INVALID_ARG);
   expect("time_next(disarm)", sdv2_profile_time_next(SDV2_KERNEL_APPEND, NULL, NULL), SDV2_OK);
-  expect("attention_stages(7)", sdv2_profile_attention_stages(7), SDV2_ERR_INVALID_ARG);
-  expect("attention_stages(all)", sdv2_profile_attention_stages(SDV2_STAGE_ALL), SDV2_OK);
   expect("copy of nothing", sdv2_copy_bytes(NULL, NULL, 0, NULL), SDV2_OK);
   printf(failures ? "FAILED: %d\n" : "all checks passed\n", failures);
   return failures ? 1 : 0;

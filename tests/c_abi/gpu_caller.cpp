@@ -71,7 +71,10 @@ int main(int argc, char** argv) {
   HIP_OK(hipMalloc(&d_len, sizeof(int32_t)));
   const size_t ws_bytes = sdv2_swa_attn_workspace_bytes(1, tokens, heads, cap, splits);
   void* d_ws = nullptr;
-  if (ws_bytes) HIP_OK(hipMalloc(&d_ws, ws_bytes));
+  if (ws_bytes) {
+    HIP_OK(hipMalloc(&d_ws, ws_bytes));
+    HIP_OK(hipMemset(d_ws, 0, ws_bytes));      // the ticket words start at zero, once
+  }
 
   const sdv2_stride3 token_major = {(int64_t)n_chunk, (int64_t)heads * 128, 128};
   const sdv2_stride3 head_major = {(int64_t)n_cache, 128, (int64_t)cap * 128};   // [heads][cap][128] in memory

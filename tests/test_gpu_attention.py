@@ -187,3 +187,79 @@ def test_full_size_properties(gpu_device, name):
     again = ops.swa_attention(q, k2, v2, lens).float()
     torch.cuda.synchronize()
     assert torch.equal(short, again)
+
+
+@pytest.mark.parametrize("rows,grid,heads,L,splits,starts", [
+    (1, (1, 6, 10), 2, 300, 1, [5]),
+    (2, (3, 4, 6), 3, 900, 2, [0, 7]),            # a chunk of three frames, rows at different frames
+    (1, (1, 30, 52), 12, 9360, 0, [57]),          # the 1.3B shape with its default split
+    (3, (2, 5, 9), 1, 1500, 3, [1021, 3, 40]),    # last frames of the table
+])
+def test_query_rotated_inside_the_kernel(gpu_device, rows, grid, heads, L, splits, starts):
+    """With a RoPE table the kernel takes the query before rotation and rotates
+    it while loading, in the append kernel's arithmetic: the output must equal,
+    bit for bit, the output for the query rotated beforehand (whose bits are
+    pinned against the oracle's complex128 product elsewhere)."""
+    from streamdiffusionv2_amd import ops, rope
+
+    torch.manual_seed(12)
+    S = grid[0] * grid[1] * grid[2]
+    q = torch.randn(rows, S, heads, 128).bfloat16()
+    k = (torch.randn(rows, heads, L, 128) * 0.5).bfloat16().to(gpu_device).permute(0, 2, 1, 3)
+    v = torch.randn(rows, heads, L, 128).bfloat16().to(gpu_device).permute(0, 2, 1, 3)
+    freqs = rope.build_freqs()
+    table = ops.device_freqs(freqs, gpu_device)
+    roped = oracle.causal_rope_apply(q, [grid] * rows, oracle.build_freqs(), starts)
+    want = ops.swa_attention(roped.to(gpu_device), k, v, None, num_splits=splits)
+    got = ops.swa_attention(q.to(gpu_device), k, v, None, num_splits=splits, rope=(table, grid[1:], starts))
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    ref = oracle.attention_fp32_reference(roped, k.cpu(), v.cpu(), [L] * rows)
+    _check(got.cpu(), ref)
+
+
+def test_rope_arguments_are_checked(gpu_device):
+    from streamdiffusionv2_amd import ops, rope
+
+    table = ops.device_freqs(rope.build_freqs(), gpu_device)
+    q = torch.zeros(1, 60, 2, 128, dtype=torch.bfloat16, device=gpu_device)
+    kv = torch.zeros(1, 128, 2, 128, dtype=torch.bfloat16, device=gpu_device)
+    with pytest.raises(RuntimeError):       # 60 tokens are not whole frames of 7 x 8
+        ops.swa_attention(q, kv, kv, None, rope=(table, (7, 8), [0]))
+    with pytest.raises(RuntimeError):       # frame beyond the table
+        ops.swa_attention(q, kv, kv, None, rope=(table, (6, 10), [1024]))
+    with pytest.raises(RuntimeError):       # one start frame per row
+        ops.swa_attention(q, kv, kv, None, rope=(table, (6, 10), [0, 1]))
+    many = torch.zeros(17, 60, 1, 128, dtype=torch.bfloat16, device=gpu_device)
+    kv17 = torch.zeros(17, 128, 1, 128, dtype=torch.bfloat16, device=gpu_device)
+    with pytest.raises(RuntimeError):       # more rows than the argument block carries start frames for
+        ops.swa_attention(many, kv17, kv17, None, rope=(table, (6, 10), [0] * 17))
+
+
+def test_one_workspace_serves_changing_shapes(gpu_device):
+    """The ticket words at the head of a split-KV workspace are left at zero by
+    every call, so one zero-filled buffer serves calls of any shape and split
+    count, one after the other, and repeated calls give identical bits."""
+    from streamdiffusionv2_amd import _capi, ops
+
+    lib = _capi.lib()
+    torch.manual_seed(13)
+    shapes = [(2, 700, 3, 2000, 3), (1, 90, 5, 3000, 5), (3, 300, 2, 1200, 2), (2, 700, 3, 2000, 3)]
+    need = max(lib.sdv2_swa_attn_workspace_bytes(r, s, h, l, sp) for r, s, h, l, sp in shapes)
+    ws = ops.new_workspace(gpu_device, need)
+    first = {}
+    for rows, S, H, L, sp in shapes:
+        gen = torch.Generator().manual_seed(rows * 1000 + S)
+        q = torch.randn(rows, S, H, 128, generator=gen).bfloat16()
+        k = torch.randn(rows, L, H, 128, generator=gen).bfloat16()
+        v = torch.randn(rows, L, H, 128, generator=gen).bfloat16()
+        got = ops.swa_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), None, num_splits=sp, workspace=ws)
+        again = ops.swa_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), None, num_splits=sp, workspace=ws)
+        torch.cuda.synchronize()
+        assert torch.equal(got, again)
+        _check(got.cpu(), oracle.attention_fp32_reference(q, k, v, [L] * rows))
+        key = (rows, S, H, L, sp)
+        if key in first:
+            assert torch.equal(got, first[key])
+        first[key] = got
+        assert not ws[:65536].any()                     # the ticket words

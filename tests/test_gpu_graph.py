@@ -49,7 +49,7 @@ class _Layer:
         self.override = torch.full((self.rows,), -1, dtype=torch.long, device=dev)
         self.refresh = torch.full((self.rows,), -7, dtype=torch.int32, device=dev)
         need = ops._capi.lib().sdv2_swa_attn_workspace_bytes(self.rows, self.tokens, self.heads, self.cap, 3)
-        self.workspace = torch.empty(need, dtype=torch.uint8, device=dev)
+        self.workspace = ops.new_workspace(dev, need)
 
     def load(self, gen):
         shape = tuple(self.q.shape)

@@ -53,7 +53,7 @@ def test_static_entry_point_matches_the_workspace_one(gpu_device):
         print(f"static scratch: rows={rows} q={q_tokens} heads={heads} keys={keys} splits={splits}", flush=True)
         q, kc, vc, seq = _case(gpu_device, gen, rows, q_tokens, heads, keys, lens)
         need = lib.sdv2_swa_attn_workspace_bytes(rows, q_tokens, heads, keys, splits)
-        ws = torch.empty(max(need, 256), dtype=torch.uint8, device=gpu_device)
+        ws = torch.zeros(max(need, 256), dtype=torch.uint8, device=gpu_device)
         want = torch.full_like(q, float("nan"))
         got = torch.full_like(q, float("nan"))
         _capi.check(lib.sdv2_swa_attn_fwd(C.byref(_attn_params(q, kc, vc, want, seq, splits, ws))), "sdv2_swa_attn_fwd")
@@ -104,7 +104,7 @@ def test_static_entry_point_at_the_wan_shapes(gpu_device):
         splits = lib.sdv2_swa_attn_default_splits(1, 1560, heads, 9360)
         need = lib.sdv2_swa_attn_workspace_bytes(1, 1560, heads, 9360, 0)
         assert splits > 1 and 0 < need <= _capi.STATIC_SCRATCH_BYTES
-        ws = torch.empty(need, dtype=torch.uint8, device=gpu_device)
+        ws = torch.zeros(need, dtype=torch.uint8, device=gpu_device)
         want, got = torch.empty_like(q), torch.empty_like(q)
         _capi.check(lib.sdv2_swa_attn_fwd(C.byref(_attn_params(q, kc, vc, want, None, 0, ws))), "sdv2_swa_attn_fwd")
         _capi.check(lib.sdv2_swa_attn_fwd_static(C.byref(_attn_params(q, kc, vc, got, None, 0))),
