@@ -270,9 +270,32 @@ typedef struct sdv2_sink_sim_params {
    * fill position whatever the queue head is, :326-337), else -1.            */
   int64_t* dst_start_override;
   uint32_t override_rows;
+  /* Optional: k_in is the raw k projection and its RMSNorm (WanRMSNorm,
+   * wan_base/modules/model.py:70-86) is folded in, as in sdv2_kv_append_rope:
+   * the weight (heads * 128 elements of the tensors' dtype) and eps.          */
+  const void* k_norm_weight;
+  float norm_eps;
+  /* Optional: token sums of the cached sink frames kept between calls
+   * (device, sdv2_sink_frame_sums_bytes(), any initial contents).  The sums of
+   * a sink frame only change when the frame is written, so a caller that
+   * brings this buffer has the call read the new chunk alone:
+   *   - stale_frames[i] (host [B]): bit j set = sink frame j of row i was
+   *     written by something other than the appends this call was told about
+   *     since its sums were last taken (or never summed): it is summed from the
+   *     cache in this call;
+   *   - planned_frame[i] (host [B]): the sink frame the append that follows
+   *     writes row i's chunk to by the caller's plan (a cache still filling,
+   *     or a queue headed by an earlier refresh), or -1.  The new chunk's sums
+   *     are then filed as that frame's; for a row flagged in override_rows
+   *     that refreshes in this call, as the refreshed frame's instead.
+   * All three NULL: every sink frame is summed from the cache, every call.    */
+  float* frame_sums;
+  const uint32_t* stale_frames;
+  const int32_t* planned_frame;
 } sdv2_sink_sim_params;
 
-size_t sdv2_sink_similarity_workspace_bytes(int32_t rows, int32_t heads, int32_t sink_frames);
+size_t sdv2_sink_similarity_workspace_bytes(int32_t rows, int32_t tokens, int32_t heads, int32_t sink_frames);
+size_t sdv2_sink_frame_sums_bytes(int32_t rows, int32_t heads, int32_t sink_frames);
 int sdv2_sink_similarity(const sdv2_sink_sim_params* p);
 
 /* ------------------------------------------------------------------------

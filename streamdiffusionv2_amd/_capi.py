@@ -40,6 +40,7 @@ EXPORTED_SYMBOLS = (
     "sdv2_swa_attn_fwd",
     "sdv2_swa_attn_fwd_static",
     "sdv2_sink_similarity_workspace_bytes",
+    "sdv2_sink_frame_sums_bytes",
     "sdv2_sink_similarity",
     "sdv2_cache_relayout",
     "sdv2_event_create",
@@ -121,6 +122,11 @@ class SinkSimParams(C.Structure):
         ("stream", C.c_void_p),
         ("dst_start_override", C.c_void_p),
         ("override_rows", C.c_uint32),
+        ("k_norm_weight", C.c_void_p),
+        ("norm_eps", C.c_float),
+        ("frame_sums", C.c_void_p),
+        ("stale_frames", C.POINTER(C.c_uint32)),
+        ("planned_frame", C.POINTER(C.c_int32)),
     ]
 
 
@@ -174,7 +180,9 @@ def lib() -> C.CDLL:
     handle.sdv2_swa_attn_fwd_static.restype = C.c_int
     handle.sdv2_swa_attn_fwd_static.argtypes = [C.POINTER(AttnParams)]
     handle.sdv2_sink_similarity_workspace_bytes.restype = C.c_size_t
-    handle.sdv2_sink_similarity_workspace_bytes.argtypes = [C.c_int32] * 3
+    handle.sdv2_sink_similarity_workspace_bytes.argtypes = [C.c_int32] * 4
+    handle.sdv2_sink_frame_sums_bytes.restype = C.c_size_t
+    handle.sdv2_sink_frame_sums_bytes.argtypes = [C.c_int32] * 3
     handle.sdv2_sink_similarity.restype = C.c_int
     handle.sdv2_sink_similarity.argtypes = [C.POINTER(SinkSimParams)]
     handle.sdv2_cache_relayout.restype = C.c_int

@@ -167,6 +167,38 @@ class RingKVPath:
         """The decision is on the host once the stream has passed this point."""
         event.record(torch.cuda.current_stream(dev))
 
+    # Token sums of the cached sink frames, kept between the adaptive checks of
+    # this path so that a check reads the new chunk only.  `stale` holds, per
+    # cache row, the sink frames whose sums have to be taken from the cache
+    # again: all of them for a new cache, and any frame written by a call that
+    # did not run the check.
+    _sink_sums = None
+
+    def forget_sink_sums(self) -> None:
+        """Call after the sink frames of this layer's cache were written behind
+        the path's back (copied over, reset, received from another owner)."""
+        self._sink_sums = None
+
+    def _kept_sink_sums(self, kv_cache, rows: int, heads: int):
+        key = (kv_cache["k"].data_ptr(), kv_cache["v"].data_ptr(), tuple(kv_cache["k"].shape), self.sink_size,
+               ring.contents_generation(kv_cache))
+        kept = self._sink_sums
+        if kept is None or kept["key"] != key or len(kept["stale"]) != rows:
+            kept = dict(key=key, stale=[(1 << self.sink_size) - 1] * rows,
+                        sums=ops.new_sink_frame_sums(rows, heads, self.sink_size, kv_cache["k"].device))
+            self._sink_sums = kept
+        return kept
+
+    def _sink_frames_written(self, kv_cache, plan, tokens: int, frame_tokens: int) -> None:
+        """A call that did not run the check wrote plan.dst_start: the kept sums
+        of the sink frames it touched are stale."""
+        kept = self._sink_sums
+        if kept is None or kept["key"][0] != kv_cache["k"].data_ptr():
+            return
+        for i, dst in enumerate(plan.dst_start[:len(kept["stale"])]):
+            for frame in range(dst // frame_tokens, min(self.sink_size, (dst + tokens - 1) // frame_tokens + 1)):
+                kept["stale"][i] |= 1 << frame
+
     def _layer_launcher(self, q, k, v, kv_cache, table, grid, qk_norm=None):
         """The cached launch descriptors for this layer, rebuilt when the
         cache, the shapes, the grid or the norm weights change."""
@@ -208,10 +240,8 @@ class RingKVPath:
         table = ops.device_freqs(freqs, q.device)
         self._last_refresh = None
         adaptive = self.sink_size * frame_tokens > 0 and self.adapt_sink_thr > -1 and q.shape[1] <= frame_tokens
+        k_norm = (qk_norm[1], qk_norm[2]) if qk_norm is not None else None
         if adaptive:
-            if qk_norm is not None:
-                raise RuntimeError("adaptive sink refresh reads the normalised key before the append: "
-                                   "apply the q/k norm outside (qk_norm=None) in this mode")
             if q.shape[1] != frame_tokens:
                 raise RuntimeError(
                     f"adaptive sink refresh needs one-frame chunks ({frame_tokens} tokens), got {q.shape[1]}"
@@ -223,7 +253,7 @@ class RingKVPath:
                 # the decision is needed before anything can be planned.
                 _, refresh = ops.sink_similarity(
                     k, v, kv_cache["k"], kv_cache["v"], table, (h, w), [c // frame_tokens for c in starts],
-                    self.sink_size, self.adapt_sink_thr)
+                    self.sink_size, self.adapt_sink_thr, k_norm=k_norm)
                 self._last_refresh = refresh.tolist()
                 for i, frame in enumerate(self._last_refresh):
                     if frame >= 0:
@@ -240,14 +270,24 @@ class RingKVPath:
             # reduction on the device, whose decision goes straight to the
             # append below and, written into pinned memory by the kernel, to the host
             override, host, event = self._decision_buffers(rows, q.device)
+            kept = self._kept_sink_sums(kv_cache, rows, q.shape[2])
+            extra = {}
+            if kept is not None:
+                # where the chunk lands by the plan, if that is a sink frame: a row still filling,
+                # or an evicting one whose queue is headed by a refresh decided while it was filling
+                planned = [d // frame_tokens if d < self.sink_size * frame_tokens else -1 for d in plan.dst_start]
+                extra = dict(frame_sums=kept["sums"], stale_frames=list(kept["stale"]), planned_frames=planned)
+                kept["stale"] = [0] * rows        # summed now, and kept current by the decision kernel from here on
             ops.sink_similarity(
                 k, v, kv_cache["k"], kv_cache["v"], table, (h, w), [c // frame_tokens for c in starts],
                 self.sink_size, self.adapt_sink_thr, dst_start_override=override, override_rows=plan.evicting,
-                refresh_out=host)
+                refresh_out=host, k_norm=k_norm, **extra)
             self._mark_decision(event, q.device)
             self._pending = dict(event=event, host=host, plan=plan, queues=queues_before, starts=list(starts),
                                  tokens=q.shape[1], frame_tokens=frame_tokens, sink_size=self.sink_size,
                                  cap=kv_cache["k"].shape[1])
+        if not adaptive:
+            self._sink_frames_written(kv_cache, plan, q.shape[1], frame_tokens)
         span = plan.max_seq_len
         seq = None
         if any(n != span for n in plan.new_local_end):
@@ -310,10 +350,11 @@ class CausalWanSelfAttention(nn.Module, RingKVPath):
         self.qk_norm = qk_norm
         self.eps = eps
 
-        # True runs the q / k RMSNorm inside the append kernel.  Off by default:
-        # its sum of squares is taken in another order than torch's, so the
-        # cache can then differ from the unfused path by one ulp in rare elements.
-        self.fuse_qk_norm = False
+        # The q / k RMSNorm runs inside the append kernel (its sum of squares in
+        # the order of torch's CPU kernel, so the cache holds the bits the
+        # reference's CPU path would store); False applies the two norms as
+        # separate torch modules before the path.
+        self.fuse_qk_norm = True
 
         # ring state, same defaults as causal_model.py:177-179
         self.sink_size = 3
@@ -350,8 +391,8 @@ class CausalWanSelfAttention(nn.Module, RingKVPath):
             )
         b, s, n, d = *x.shape[:2], self.num_heads, self.head_dim
         v = self.v(x).view(b, s, n, d)
-        adaptive = self.sink_size > 0 and self.adapt_sink_thr > -1
-        if self.qk_norm and self.fuse_qk_norm and not adaptive:
+        if self.qk_norm and self.fuse_qk_norm and x.dtype in (torch.bfloat16, torch.float32) \
+                and self.num_heads <= 64:
             # the two RMSNorms run inside the append kernel
             q, k = self.q(x).view(b, s, n, d), self.k(x).view(b, s, n, d)
             norm = (self.norm_q.weight.detach(), self.norm_k.weight.detach(), self.eps)

@@ -129,24 +129,16 @@ void kv_append_rope_kernel(const AppendKernelArgs a) {
 // causal_model.py:212-218): y = type_as(x.float() * rsqrt(mean(x^2) + eps)) *
 // weight over the full heads * 128 vector of a token, then RoPE and the
 // scatter as above.  One wave per token: lane l owns the 8-element slice
-// l % 16 of heads 4 * j + l / 16 (j = 0, 1, ...), keeps its q / k slices in
-// registers between the sum of squares and the write, and the wave reduces the
-// two sums with cross-lane adds in a fixed order.  Rounding steps are the
+// l % 16 of heads 4 * j + l / 16 (j = 0, 1, ...) and keeps its q / k slices in
+// registers between the sum of squares and the write.  Rounding steps are the
 // reference's: normalised value to the storage type, times weight to the
 // storage type, rotation in double to float to the storage type.
+//
+// The sum of squares is taken in the order of PyTorch's CPU sum kernel
+// (sdv2::wave_sum_squares), so that mean, rsqrt and everything after them come
+// out bit for bit as on the reference's CPU path.
 // ---------------------------------------------------------------------------
 constexpr int kNormMaxSteps = 16;           // heads <= 64
-
-template <typename T>
-__device__ __forceinline__ sdv2::Vec8<T> normalise(const sdv2::Vec8<T>& x, float r, const sdv2::Vec8<T>& w) {
-  sdv2::Vec8<T> y;
-  sdv2::Vec8<T> n;                           // x * r in the storage type
-#pragma unroll
-  for (int p = 0; p < 4; ++p) n.setf_pair(p, x.getf(2 * p) * r, x.getf(2 * p + 1) * r);
-#pragma unroll
-  for (int p = 0; p < 4; ++p) y.setf_pair(p, n.getf(2 * p) * w.getf(2 * p), n.getf(2 * p + 1) * w.getf(2 * p + 1));
-  return y;
-}
 
 template <typename T, int kSteps>
 __global__ __launch_bounds__(256)
@@ -181,7 +173,6 @@ void kv_append_norm_rope_kernel(const AppendKernelArgs a) {
   const int steps = (a.heads + 3) >> 2;
 
   sdv2::Vec8<T> q[kSteps], k[kSteps];
-  float ssq_q = 0.f, ssq_k = 0.f;
 #pragma unroll
   for (int j = 0; j < kSteps; ++j) {
     const int h = 4 * j + head_in_step;
@@ -189,18 +180,14 @@ void kv_append_norm_rope_kernel(const AppendKernelArgs a) {
       q[j] = sdv2::Vec8<T>::load(qi + h * a.q_in_st.head);
       k[j] = sdv2::Vec8<T>::load(ki + h * a.k_in_st.head);
       sdv2::Vec8<T>::load(vi + h * a.v_in_st.head).store(vc + h * a.v_st.head);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        ssq_q += q[j].getf(i) * q[j].getf(i);
-        ssq_k += k[j].getf(i) * k[j].getf(i);
-      }
+    } else {
+      q[j] = sdv2::Vec8<T>::zero();
+      k[j] = sdv2::Vec8<T>::zero();
     }
   }
-#pragma unroll
-  for (int off = 1; off < 64; off <<= 1) {
-    ssq_q += __shfl_xor(ssq_q, off, 64);
-    ssq_k += __shfl_xor(ssq_k, off, 64);
-  }
+  __shared__ float squares[4][2][64 * 8];          // per wave: one step's squares of k and of q
+  float ssq_k, ssq_q;
+  sdv2::wave_sum_squares<T, kSteps>(k, q, a.heads, squares[threadIdx.x >> 6], lane, ssq_k, ssq_q);
   const float width = static_cast<float>(a.heads * 128);
   const float rq = 1.0f / sqrtf(ssq_q / width + a.norm_eps);
   const float rk = 1.0f / sqrtf(ssq_k / width + a.norm_eps);
@@ -210,8 +197,8 @@ void kv_append_norm_rope_kernel(const AppendKernelArgs a) {
   for (int j = 0; j < kSteps; ++j) {
     const int h = 4 * j + head_in_step;
     if (j < steps && h < a.heads) {
-      const sdv2::Vec8<T> qn = normalise(q[j], rq, sdv2::Vec8<T>::load(wq + h * 128));
-      const sdv2::Vec8<T> kn = normalise(k[j], rk, sdv2::Vec8<T>::load(wk + h * 128));
+      const sdv2::Vec8<T> qn = sdv2::normalise(q[j], rq, sdv2::Vec8<T>::load(wq + h * 128));
+      const sdv2::Vec8<T> kn = sdv2::normalise(k[j], rk, sdv2::Vec8<T>::load(wk + h * 128));
       sdv2::rotate(qn, cs).store(qo + h * a.q_out_st.head);
       sdv2::rotate(kn, cs).store(kc + h * a.k_st.head);
     }

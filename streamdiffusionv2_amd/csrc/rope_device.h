@@ -17,6 +17,11 @@ struct Vec8;
 template <>
 struct Vec8<uint16_t> {                     // bf16 bit patterns
   uint4 raw;
+  __device__ static Vec8 zero() {
+    Vec8 v;
+    v.raw = make_uint4(0u, 0u, 0u, 0u);
+    return v;
+  }
   __device__ static Vec8 load(const uint16_t* p) {
     Vec8 v;
     v.raw = *reinterpret_cast<const uint4*>(p);
@@ -44,6 +49,12 @@ struct Vec8<uint16_t> {                     // bf16 bit patterns
 template <>
 struct Vec8<float> {
   float4 lo, hi;
+  __device__ static Vec8 zero() {
+    Vec8 v;
+    v.lo = make_float4(0.f, 0.f, 0.f, 0.f);
+    v.hi = v.lo;
+    return v;
+  }
   __device__ static Vec8 load(const float* p) {
     Vec8 v;
     v.lo = *reinterpret_cast<const float4*>(p);
@@ -99,6 +110,80 @@ __device__ __forceinline__ void load_rotation(const double2* freqs, int pairs, i
     const int64_t pos = p < split_t ? frame : (p < split_h ? hi : wi);
     cs[j] = freqs[pos * pairs + p];
   }
+}
+
+// WanRMSNorm of an 8-element slice once the token's 1 / rms is known
+// (wan_base/modules/model.py:77-86): x * r rounded to the storage type, times
+// the weight, rounded to the storage type again.
+template <typename T>
+__device__ __forceinline__ Vec8<T> normalise(const Vec8<T>& x, float r, const Vec8<T>& w) {
+  Vec8<T> y;
+  Vec8<T> n;                           // x * r in the storage type
+#pragma unroll
+  for (int p = 0; p < 4; ++p) n.setf_pair(p, x.getf(2 * p) * r, x.getf(2 * p + 1) * r);
+#pragma unroll
+  for (int p = 0; p < 4; ++p) y.setf_pair(p, n.getf(2 * p) * w.getf(2 * p), n.getf(2 * p + 1) * w.getf(2 * p + 1));
+  return y;
+}
+
+// Sum of squares of a token's full heads * 128 vector, for two vectors at once
+// (k and q), by one wave, in the order of PyTorch's CPU sum kernel (ATen
+// cascade_sum / vectorized_inner_sum with 8-float vectors, which the AVX2 and
+// AVX512 builds share): element e of the row belongs to accumulator (e / 8 % 4,
+// e % 8); an accumulator adds its elements in blocks of 16, each block summed
+// in order from zero, the block sums added up in order; a trailing partial
+// block goes first; then the four accumulators of a vector lane are added in
+// order, then the eight lanes in order, starting from zero.  The caller has
+// checked this against torch bit for bit on the CPU.
+//
+// Lane l of the wave holds, per step j, the slice l % 16 of head 4 j + l / 16
+// (zeros past the last head).  With e = 128 head + 8 slice + t the 16 lanes
+// l % 4 == c of a step hold exactly one block of accumulator (c, t), in lane
+// order.  Per step every lane parks its 8 + 8 squares in `scratch` (2 x 512
+// floats of this wave) and lanes 0-31 (k) / 32-63 (q) each walk one
+// accumulator's block; LDS operations of a wave complete in order, so no
+// barrier is needed.
+template <typename T, int kSteps>
+__device__ __forceinline__ void wave_sum_squares(const Vec8<T> (&k)[kSteps], const Vec8<T> (&q)[kSteps], int heads,
+                                                 float (&scratch)[2][64 * 8], int lane, float& sum_k, float& sum_q) {
+#pragma clang fp contract(off)
+  const int which = lane >> 5;               // lanes 0-31 add up k, lanes 32-63 q
+  const int chain = lane & 31;               // accumulator (c, t) = (chain % 4, chain / 4)
+  const int c = chain & 3, t = chain >> 2;
+  const int full = heads >> 2;               // steps whose four heads all exist: whole blocks of 16
+  const int tail = 4 * (heads & 3);          // elements of the trailing partial block
+  float blocks = 0.f;                        // the whole blocks' sums, added up in order
+  float trailing = 0.f;
+#pragma unroll
+  for (int j = 0; j < kSteps; ++j) {
+    if (4 * j < heads) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        scratch[0][lane * 8 + i] = k[j].getf(i) * k[j].getf(i);
+        scratch[1][lane * 8 + i] = q[j].getf(i) * q[j].getf(i);
+      }
+      const int count = j < full ? 16 : tail;
+      float block = 0.f;
+#pragma unroll
+      for (int m = 0; m < 16; ++m)
+        if (m < count) block += scratch[which][(c + 4 * m) * 8 + t];
+      if (j < full) blocks += block;
+      else trailing = block;
+    }
+  }
+  const float mine = tail ? trailing + blocks : blocks;
+  // the four accumulators of vector lane t, in order (they sit in neighbouring lanes)
+  const int quad = lane & ~3;
+  float lane_sum = __shfl(mine, quad, 64);
+  lane_sum += __shfl(mine, quad + 1, 64);
+  lane_sum += __shfl(mine, quad + 2, 64);
+  lane_sum += __shfl(mine, quad + 3, 64);
+  // the eight vector lanes, in order, from zero
+  float total = 0.f;
+#pragma unroll
+  for (int v = 0; v < 8; ++v) total += __shfl(lane_sum, (lane & 32) + 4 * v, 64);
+  sum_k = __shfl(total, 0, 64);
+  sum_q = __shfl(total, 32, 64);
 }
 
 }  // namespace sdv2

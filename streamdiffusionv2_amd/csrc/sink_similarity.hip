@@ -20,8 +20,20 @@
 // two cosine similarities and their sum are each rounded to bf16 (they are
 // bf16 tensors in the reference); sums inside a reduction are fp32 in a fixed
 // order, so results are deterministic.
+//
+// The sums of the cached sink frames only change when a sink frame is written.
+// A caller that keeps them between calls (frame_sums) has the reduction read
+// the new chunk alone: the decision kernel files the new chunk's sums under the
+// sink frame the append that follows will overwrite, and only frames the
+// caller marks stale are summed from the cache again.
+//
+// When the q / k RMSNorm is folded into the append the keys arrive raw: a
+// first small kernel then takes every token's 1 / rms (in the append's
+// arithmetic) and the reduction normalises before it rotates.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 #include "sdv2kv.h"
 #include "sdv2kv_profile.h"
@@ -43,7 +55,13 @@ struct SinkSimKernelArgs {
   const void* v_cache;
   sdv2_stride3 k_in_st, v_in_st, k_st, v_st;
   const double2* freqs;
-  float* sums;                              // [rows][2*sink+2][heads*128][kTokenSplits]: token sums
+  float* sums;                              // [rows][2*sink+2][heads*128][kTokenSplits]: token sums of this call
+  float* kept;                              // [rows][2*sink][heads*128][kTokenSplits] kept between calls, or null
+  const void* k_norm_w;                     // RMSNorm weight of k over heads * 128, or null
+  float* inv_rms;                           // [rows][tokens]: 1 / rms of every new key token (with k_norm_w)
+  float norm_eps;
+  uint32_t stale[SDV2_MAX_ROWS];            // bit j: sink frame j of the row is summed from the cache in this call
+  int32_t planned_frame[SDV2_MAX_ROWS];     // sink frame the host's plan writes this call's chunk to, or -1
   float* similarity;                        // [rows][sink]
   int32_t* refresh;                         // [rows]
   int64_t* dst_override;                    // [rows] or null: slot start for the append that follows
@@ -53,6 +71,14 @@ struct SinkSimKernelArgs {
   float threshold;
   int64_t start_frame[SDV2_MAX_ROWS];
 };
+
+// where the token sums of matrix m (sink K frames, sink V frames, new K, new V) of a row live
+__device__ __forceinline__ float* sums_of(const SinkSimKernelArgs& a, int row, int m) {
+  const int64_t width = static_cast<int64_t>(a.heads) * 128 * kTokenSplits;
+  const int sink = a.sink_frames;
+  if (a.kept && m < 2 * sink) return a.kept + (static_cast<int64_t>(row) * 2 * sink + m) * width;
+  return a.sums + (static_cast<int64_t>(row) * (2 * sink + 2) + m) * width;
+}
 
 template <typename T>
 __device__ __forceinline__ float round_to_storage(float x);
@@ -82,6 +108,8 @@ void sink_frame_sum_kernel(const SinkSimKernelArgs a) {
   const bool is_new = m >= 2 * sink;
   const bool is_k = is_new ? (m == 2 * sink) : (m < sink);
   const int frame = is_new ? 0 : (m < sink ? m : m - sink);
+  // a kept frame sum stands until the caller calls it stale
+  if (!is_new && a.kept && !((a.stale[row] >> frame) & 1u)) return;
   const sdv2_stride3 st = is_new ? (is_k ? a.k_in_st : a.v_in_st) : (is_k ? a.k_st : a.v_st);
   const T* base = static_cast<const T*>(is_new ? (is_k ? a.k_in : a.v_in) : (is_k ? a.k_cache : a.v_cache));
   base += row * st.row + static_cast<int64_t>(frame) * a.tokens * st.token + head * st.head + lane * 8;
@@ -96,6 +124,12 @@ void sink_frame_sum_kernel(const SinkSimKernelArgs a) {
       const int hi = t / a.grid_w;
       sdv2::load_rotation(a.freqs, a.pairs, a.split_t, a.split_h, lane, a.start_frame[row], hi, t - hi * a.grid_w, cs);
     };
+    // with the norm folded in: the key as the append will normalise it (same two roundings)
+    sdv2::Vec8<T> weight;
+    if (a.k_norm_w) weight = sdv2::Vec8<T>::load(static_cast<const T*>(a.k_norm_w) + head * 128 + lane * 8);
+    auto normalised = [&](const sdv2::Vec8<T>& x, int t) {
+      return sdv2::normalise(x, a.inv_rms[static_cast<int64_t>(row) * a.tokens + t], weight);
+    };
     int t = split * per + tl;
     for (; t + (kUnroll - 1) * kTokenLanes < t_end; t += kUnroll * kTokenLanes) {
       sdv2::Vec8<T> x[kUnroll];
@@ -107,6 +141,7 @@ void sink_frame_sum_kernel(const SinkSimKernelArgs a) {
       }
 #pragma unroll
       for (int u = 0; u < kUnroll; ++u) {
+        if (a.k_norm_w) x[u] = normalised(x[u], t + u * kTokenLanes);
         const sdv2::Vec8<T> y = sdv2::rotate(x[u], cs[u]);
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[i] += static_cast<float>(y.get(i));
@@ -115,7 +150,9 @@ void sink_frame_sum_kernel(const SinkSimKernelArgs a) {
     for (; t < t_end; t += kTokenLanes) {
       double2 cs[4];
       rotation(t, cs);
-      const sdv2::Vec8<T> y = sdv2::rotate(sdv2::Vec8<T>::load(base + t * st.token), cs);
+      sdv2::Vec8<T> x = sdv2::Vec8<T>::load(base + t * st.token);
+      if (a.k_norm_w) x = normalised(x, t);
+      const sdv2::Vec8<T> y = sdv2::rotate(x, cs);
 #pragma unroll
       for (int i = 0; i < 8; ++i) acc[i] += static_cast<float>(y.get(i));
     }
@@ -144,11 +181,34 @@ void sink_frame_sum_kernel(const SinkSimKernelArgs a) {
     float s = 0.f;
 #pragma unroll
     for (int j = 0; j < kTokenLanes; ++j) s += part[j][threadIdx.x];
-    const int64_t width = static_cast<int64_t>(a.heads) * 128;
     // the token ranges of one column sit side by side, so the decision kernel fetches them with two 16-byte loads
-    a.sums[((static_cast<int64_t>(row) * (2 * sink + 2) + m) * width + head * 128 + threadIdx.x) * kTokenSplits +
-           split] = s;
+    sums_of(a, row, m)[static_cast<int64_t>(head * 128 + threadIdx.x) * kTokenSplits + split] = s;
   }
+}
+
+// grid (tokens / 4, 1, rows): one wave per new key token takes 1 / sqrt(mean(k^2) + eps)
+// over the token's heads * 128 values, exactly as the append kernel with the
+// norm folded in does (same order of additions, same operations).
+template <typename T, int kSteps>
+__global__ __launch_bounds__(256)
+void key_inv_rms_kernel(const SinkSimKernelArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int tok = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int row = blockIdx.z;
+  if (tok >= a.tokens) return;
+  const T* ki = static_cast<const T*>(a.k_in) + row * a.k_in_st.row + tok * a.k_in_st.token + (lane & 15) * 8;
+  sdv2::Vec8<T> k[kSteps];
+#pragma unroll
+  for (int j = 0; j < kSteps; ++j) {
+    const int h = 4 * j + (lane >> 4);
+    k[j] = 4 * j < a.heads && h < a.heads ? sdv2::Vec8<T>::load(ki + h * a.k_in_st.head) : sdv2::Vec8<T>::zero();
+  }
+  __shared__ float squares[4][2][64 * 8];
+  float ssq_k, unused;
+  sdv2::wave_sum_squares<T, kSteps>(k, k, a.heads, squares[threadIdx.x >> 6], lane, ssq_k, unused);
+  if (lane == 0)
+    a.inv_rms[static_cast<int64_t>(row) * a.tokens + tok] =
+        1.0f / sqrtf(ssq_k / static_cast<float>(a.heads * 128) + a.norm_eps);
 }
 
 // grid (rows): frame means from the partial sums, cosine similarities, their
@@ -167,7 +227,6 @@ void sink_decide_kernel(const SinkSimKernelArgs a) {
   const int row = blockIdx.x;
   const int sink = a.sink_frames;
   const int width = a.heads * 128;
-  const float* sums = a.sums + static_cast<int64_t>(row) * (2 * sink + 2) * kTokenSplits * width;
   const float inv_tokens = 1.0f / static_cast<float>(a.tokens);
   constexpr float kEps = 1e-8f;             // torch.cosine_similarity default
   int col[kCols];
@@ -180,7 +239,7 @@ void sink_decide_kernel(const SinkSimKernelArgs a) {
   }
   // means of frame m at this thread's columns: the token ranges in order, then the rounding of a stored mean
   auto means = [&](int m, float (&out)[kCols]) {
-    const float* p = sums + static_cast<int64_t>(m) * kTokenSplits * width;
+    const float* p = sums_of(a, row, m);
     float4 part[kCols][kTokenSplits / 4];
 #pragma unroll
     for (int i = 0; i < kCols; ++i)
@@ -258,11 +317,29 @@ void sink_decide_kernel(const SinkSimKernelArgs a) {
       }
     const int frame = best < round_to_storage<T>(a.threshold) ? best_frame : -1;
     a.refresh[row] = frame;
+    sims[0] = __int_as_float(frame);          // (for the hand-over of the kept sums below)
     // The refreshed sink frame goes to the head of the row's eviction queue
     // (causal_model.py:297-299); a call on the evict branch then writes its
     // one-frame chunk at [(frame + 1) * tokens - tokens, (frame + 1) * tokens).
     if (a.dst_override)
       a.dst_override[row] = frame >= 0 && ((a.override_rows >> row) & 1u) ? static_cast<int64_t>(frame) * a.tokens : -1;
+  }
+  if (a.kept) {
+    // The append that follows overwrites a sink frame when the row evicts into
+    // the frame just chosen, or when the host's plan (a filling call) lands
+    // there: the new chunk's sums become that frame's kept sums.
+    __syncthreads();
+    const int chosen = __float_as_int(sims[0]);
+    const bool evicting = (a.override_rows >> row) & 1u;
+    const int target = evicting && a.dst_override && chosen >= 0 ? chosen : a.planned_frame[row];
+    if (target >= 0 && target < sink) {
+      const int64_t n4 = static_cast<int64_t>(width) * kTokenSplits / 4;
+      for (int which = 0; which < 2; ++which) {
+        const float4* src = reinterpret_cast<const float4*>(sums_of(a, row, 2 * sink + which));
+        float4* dst = reinterpret_cast<float4*>(sums_of(a, row, which * sink + target));
+        for (int64_t i = threadIdx.x; i < n4; i += kDecideThreads) dst[i] = src[i];
+      }
+    }
   }
 }
 
@@ -272,12 +349,23 @@ bool stride_ok(const sdv2_stride3& s, int vec) {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
-}  // namespace
-
-extern "C" size_t sdv2_sink_similarity_workspace_bytes(int32_t rows, int32_t heads, int32_t sink_frames) {
-  if (rows <= 0 || heads <= 0 || sink_frames <= 0) return 0;
+size_t sums_bytes(int32_t rows, int32_t heads, int32_t sink_frames) {
   return static_cast<size_t>(rows) * (2 * static_cast<size_t>(sink_frames) + 2) * kTokenSplits * heads * SDV2_HEAD_DIM *
          sizeof(float);
+}
+
+}  // namespace
+
+extern "C" size_t sdv2_sink_similarity_workspace_bytes(int32_t rows, int32_t tokens, int32_t heads,
+                                                        int32_t sink_frames) {
+  if (rows <= 0 || tokens <= 0 || heads <= 0 || sink_frames <= 0) return 0;
+  // token sums of every matrix of the call, then 1 / rms per new key token (used with the norm folded in)
+  return sums_bytes(rows, heads, sink_frames) + static_cast<size_t>(rows) * tokens * sizeof(float);
+}
+
+extern "C" size_t sdv2_sink_frame_sums_bytes(int32_t rows, int32_t heads, int32_t sink_frames) {
+  if (rows <= 0 || heads <= 0 || sink_frames <= 0) return 0;
+  return static_cast<size_t>(rows) * 2 * sink_frames * kTokenSplits * heads * SDV2_HEAD_DIM * sizeof(float);
 }
 
 extern "C" int sdv2_sink_similarity(const sdv2_sink_sim_params* p) {
@@ -304,15 +392,26 @@ extern "C" int sdv2_sink_similarity(const sdv2_sink_sim_params* p) {
   if (p->grid_h > p->freq_rows || p->grid_w > p->freq_rows) return SDV2_ERR_OUT_OF_RANGE;
   for (int i = 0; i < p->rows; ++i)
     if (p->start_frame[i] < 0 || p->start_frame[i] >= p->freq_rows) return SDV2_ERR_OUT_OF_RANGE;
-  const size_t need = sdv2_sink_similarity_workspace_bytes(p->rows, p->heads, p->sink_frames);
+  const size_t need = sdv2_sink_similarity_workspace_bytes(p->rows, p->tokens, p->heads, p->sink_frames);
   if (!p->workspace || p->workspace_bytes < need || (reinterpret_cast<uintptr_t>(p->workspace) & 15))
     return SDV2_ERR_WORKSPACE;
+  if (p->k_norm_weight && (!aligned16(p->k_norm_weight) || !(p->norm_eps >= 0.f))) return SDV2_ERR_INVALID_ARG;
+  if (p->frame_sums) {
+    if (reinterpret_cast<uintptr_t>(p->frame_sums) & 15) return SDV2_ERR_INVALID_ARG;
+    if (!p->stale_frames || !p->planned_frame) return SDV2_ERR_INVALID_ARG;
+    for (int i = 0; i < p->rows; ++i)
+      if (p->planned_frame[i] < -1 || p->planned_frame[i] >= p->sink_frames) return SDV2_ERR_OUT_OF_RANGE;
+  }
 
   SinkSimKernelArgs a{};
   a.k_in = p->k_in; a.v_in = p->v_in; a.k_cache = p->k_cache; a.v_cache = p->v_cache;
   a.k_in_st = p->k_in_stride; a.v_in_st = p->v_in_stride; a.k_st = p->k_cache_stride; a.v_st = p->v_cache_stride;
   a.freqs = reinterpret_cast<const double2*>(p->freqs);
   a.sums = static_cast<float*>(p->workspace);
+  a.inv_rms = reinterpret_cast<float*>(static_cast<char*>(p->workspace) + sums_bytes(p->rows, p->heads, p->sink_frames));
+  a.kept = p->frame_sums;
+  a.k_norm_w = p->k_norm_weight;
+  a.norm_eps = p->norm_eps;
   a.similarity = p->similarity;
   a.refresh = p->refresh;
   a.dst_override = p->dst_start_override;
@@ -323,15 +422,31 @@ extern "C" int sdv2_sink_similarity(const sdv2_sink_sim_params* p) {
   a.split_t = a.pairs - 2 * third;
   a.split_h = a.split_t + third;
   a.threshold = p->threshold;
-  for (int i = 0; i < p->rows; ++i) a.start_frame[i] = p->start_frame[i];
+  for (int i = 0; i < p->rows; ++i) {
+    a.start_frame[i] = p->start_frame[i];
+    a.stale[i] = p->frame_sums ? p->stale_frames[i] : 0xffffffffu;
+    a.planned_frame[i] = p->frame_sums ? p->planned_frame[i] : -1;
+  }
 
   hipStream_t stream = static_cast<hipStream_t>(p->stream);
   const dim3 block(kLanesPerRow * kTokenLanes);
   const dim3 grid_mean(p->heads, 2 * p->sink_frames + 2, p->rows * kTokenSplits);
   const dim3 grid_decide(p->rows);
+  const dim3 decide_block(kDecideThreads);
   // columns per thread of the decision kernel: 2 up to 16 heads, 8 up to 64
   const bool wide = p->heads * 128 > 2 * kDecideThreads;
-  const dim3 decide_block(kDecideThreads);
+  if (p->k_norm_weight) {
+    const dim3 grid_rms((p->tokens + 3) / 4, 1, p->rows);
+    const int steps = (p->heads + 3) / 4;
+    auto launch = [&](auto steps_c) {
+      constexpr int kS = decltype(steps_c)::value;
+      if (p->dtype == SDV2_BF16) hipLaunchKernelGGL((key_inv_rms_kernel<uint16_t, kS>), grid_rms, dim3(256), 0, stream, a);
+      else hipLaunchKernelGGL((key_inv_rms_kernel<float, kS>), grid_rms, dim3(256), 0, stream, a);
+    };
+    if (steps <= 4) launch(std::integral_constant<int, 4>{});
+    else if (steps <= 10) launch(std::integral_constant<int, 10>{});
+    else launch(std::integral_constant<int, 16>{});
+  }
   if (p->dtype == SDV2_BF16) {
     sdv2::launch_timed(SDV2_KERNEL_SINK_SUM, sink_frame_sum_kernel<uint16_t>, grid_mean, block, 0, stream, a);
     if (wide) sdv2::launch_timed(SDV2_KERNEL_SINK_DECIDE, sink_decide_kernel<uint16_t, 8>, grid_decide, decide_block, 0, stream, a);

@@ -397,6 +397,10 @@ def sink_similarity(
     dst_start_override: Optional[torch.Tensor] = None,
     override_rows: Sequence[bool] = (),
     refresh_out: Optional[torch.Tensor] = None,
+    k_norm: Optional[Tuple[torch.Tensor, float]] = None,
+    frame_sums: Optional[torch.Tensor] = None,
+    stale_frames: Sequence[int] = (),
+    planned_frames: Sequence[int] = (),
 ):
     """Adaptive sink refresh decision (causal_model.py:284-299) for a
     one-frame chunk, before its append.
@@ -408,6 +412,16 @@ def sink_similarity(
     decision instead of a new device tensor; it may be PINNED host memory, which
     the kernel then writes directly (valid on the host once the stream has
     passed this call).
+
+    ``k_norm`` = (k norm weight, eps): k is the raw k projection and its
+    RMSNorm is applied inside, as :func:`kv_append_rope` with ``qk_norm`` does.
+
+    ``frame_sums`` (from :func:`new_sink_frame_sums`) keeps the token sums of
+    the cached sink frames between calls, so that only the new chunk is read:
+    ``stale_frames[i]`` is a bit mask of the sink frames of row i whose sums
+    must be taken from the cache again (written behind this operator's back,
+    or never summed), ``planned_frames[i]`` the sink frame the append that
+    follows writes to by the host's plan, or -1.
 
     k is the chunk's key BEFORE RoPE, v its value, both [B,S,H,128]; the caches
     are read as they are.  Returns (similarity float32 [B, sink_frames],
@@ -423,7 +437,7 @@ def sink_similarity(
     if k_cache.shape[0] < rows or v_cache.shape != k_cache.shape or k_cache.shape[2] != heads:
         raise RuntimeError(f"cache {tuple(k_cache.shape)} does not match the chunk {tuple(k.shape)}")
     lib = _capi.lib()
-    need = lib.sdv2_sink_similarity_workspace_bytes(rows, heads, sink_frames)
+    need = lib.sdv2_sink_similarity_workspace_bytes(rows, tokens, heads, sink_frames)
     ws = _SIM_WORKSPACES.get(dev)
     if ws is None or ws.numel() < need:
         ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
@@ -462,9 +476,34 @@ def sink_similarity(
             raise RuntimeError("override_rows needs one flag per row")
         p.dst_start_override = dst_start_override.data_ptr()
         p.override_rows = sum(1 << i for i, flag in enumerate(override_rows) if flag)
+    if k_norm is not None:
+        weight, eps = k_norm
+        if weight.dtype != k.dtype or weight.numel() != heads * HEAD_DIM or not weight.is_contiguous() \
+                or weight.device != dev:
+            raise RuntimeError(f"the k norm weight must be a contiguous {k.dtype} tensor of {heads * HEAD_DIM} elements on {dev}")
+        p.k_norm_weight, p.norm_eps = weight.data_ptr(), float(eps)
+    if frame_sums is not None:
+        want = lib.sdv2_sink_frame_sums_bytes(rows, heads, sink_frames)
+        if frame_sums.device != dev or not frame_sums.is_contiguous() \
+                or frame_sums.numel() * frame_sums.element_size() < want:
+            raise RuntimeError(f"frame_sums must be a contiguous buffer of at least {want} bytes on {dev}")
+        if len(stale_frames) != rows or len(planned_frames) != rows:
+            raise RuntimeError("frame_sums needs stale_frames and planned_frames with one entry per row")
+        stale = (C.c_uint32 * rows)(*[int(x) & 0xffffffff for x in stale_frames])
+        planned = (C.c_int32 * rows)(*[int(x) for x in planned_frames])
+        p.frame_sums = frame_sums.data_ptr()
+        p.stale_frames = C.cast(stale, C.POINTER(C.c_uint32))
+        p.planned_frame = C.cast(planned, C.POINTER(C.c_int32))
     with torch.cuda.device(dev):
         _capi.check(lib.sdv2_sink_similarity(C.byref(p)), "sdv2_sink_similarity")
     return similarity, refresh
+
+
+def new_sink_frame_sums(rows: int, heads: int, sink_frames: int, dev) -> torch.Tensor:
+    """The buffer :func:`sink_similarity` keeps the sink frames' token sums in
+    between calls (everything in it starts out stale)."""
+    n = _capi.lib().sdv2_sink_frame_sums_bytes(rows, heads, sink_frames)
+    return torch.empty(max(n // 4, 1), dtype=torch.float32, device=dev)
 
 
 class KernelTimer:

@@ -27,6 +27,7 @@ import torch
 
 HEAD_DIM = 128
 _MIRROR_KEY = "_sdv2_host_index_mirror"
+_GENERATION_KEY = "_sdv2_contents_generation"
 
 
 def tensor_version(t: torch.Tensor) -> Optional[int]:
@@ -147,10 +148,25 @@ def rows_evicting(kv_cache: dict, current_start: Sequence[int], n_new: int) -> L
 
 
 def forget_index_mirror(kv_cache: dict) -> None:
-    """Drop the host copy of the two index tensors.  Needed after the library
-    itself rewrote them on the device (a raw kernel store does not bump the
-    tensors' version counters); the next plan reads them back once."""
+    """Drop what the host remembers about this cache: its copy of the two
+    index tensors (the next plan reads them back once) and, through
+    :func:`contents_changed`, every layer path's kept sums of the sink frames.
+    Needed after the tensors of the dict were rewritten in place by anything
+    but the path's own calls - the library's hand-off kernel, a copy between
+    rows, a reset (a raw device store bumps no version counter, and tensors
+    created under ``torch.inference_mode()`` have none)."""
     kv_cache.pop(_MIRROR_KEY, None)
+    contents_changed(kv_cache)
+
+
+def contents_changed(kv_cache: dict) -> None:
+    """Tell the paths that read this cache that k / v rows changed behind
+    their back (see :func:`forget_index_mirror`)."""
+    kv_cache[_GENERATION_KEY] = kv_cache.get(_GENERATION_KEY, 0) + 1
+
+
+def contents_generation(kv_cache: dict) -> int:
+    return kv_cache.get(_GENERATION_KEY, 0)
 
 
 @dataclass

@@ -220,6 +220,7 @@ class KVStreamPipeline:
                 if t.shape[0] > 1 and t.stride(0) != 0:
                     t[1:].copy_(t[:1].expand_as(t[1:]))
                 entry[name] = t
+            ring.contents_changed(entry)       # rows rewritten here: kept sums of the sink frames are stale
             if "total_steps" in entry:
                 entry["current_step"] = entry["total_steps"]
         self.hidden_states = torch.zeros_like(self._batch_state_refs["hidden_states"])

@@ -72,15 +72,15 @@ int main(void) {
          offsetof(sdv2_append_params, stream), offsetof(sdv2_append_params, dst_start_override));
   printf("layout sdv2_attn_params size=%zu stream=%zu rope_start_frame=%zu\n", sizeof(sdv2_attn_params),
          offsetof(sdv2_attn_params, stream), offsetof(sdv2_attn_params, rope_start_frame));
-  printf("layout sdv2_sink_sim_params size=%zu stream=%zu override_rows=%zu\n", sizeof(sdv2_sink_sim_params),
-         offsetof(sdv2_sink_sim_params, stream), offsetof(sdv2_sink_sim_params, override_rows));
+  printf("layout sdv2_sink_sim_params size=%zu stream=%zu planned_frame=%zu\n", sizeof(sdv2_sink_sim_params),
+         offsetof(sdv2_sink_sim_params, stream), offsetof(sdv2_sink_sim_params, planned_frame));
   printf("layout sdv2_relayout_params size=%zu stream=%zu global_end_shift=%zu\n", sizeof(sdv2_relayout_params),
          offsetof(sdv2_relayout_params, stream), offsetof(sdv2_relayout_params, global_end_shift));
 
   printf("splits for 1x1560 tokens, 12 heads, 9360 keys: %d\n", sdv2_swa_attn_default_splits(1, 1560, 12, 9360));
   printf("workspace for that call: %zu bytes\n", sdv2_swa_attn_workspace_bytes(1, 1560, 12, 9360, 0));
   printf("sink-similarity workspace, 1 row, 12 heads, 3 sink frames: %zu bytes\n",
-         sdv2_sink_similarity_workspace_bytes(1, 12, 3));
+         sdv2_sink_similarity_workspace_bytes(1, 1560, 12, 3));
   expect("attention_static(NULL)", sdv2_swa_attn_fwd_static(NULL), SDV2_ERR_INVALID_ARG);
   expect("event_create(NULL)", sdv2_event_create(NULL), SDV2_ERR_INVALID_ARG);
   expect("time_next(unknown kernel)", sdv2_profile_time_next(SDV2_KERNEL_COUNT, NULL, NULL), SDV2_ERR_INVALID_ARG);

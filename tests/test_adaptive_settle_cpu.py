@@ -65,7 +65,7 @@ def _patched_path(monkeypatch, script, sink):
     calls = {"n": 0}
 
     def fake_similarity(k, v, k_cache, v_cache, table, grid_hw, start_frames, sink_frames, threshold,
-                        dst_start_override=None, override_rows=(), refresh_out=None):
+                        dst_start_override=None, override_rows=(), refresh_out=None, **kept):
         decisions = script[calls["n"]]
         calls["n"] += 1
         rows = k.shape[0]
@@ -80,6 +80,7 @@ def _patched_path(monkeypatch, script, sink):
     monkeypatch.setattr(attention.ops, "sink_similarity", fake_similarity)
     monkeypatch.setattr(path, "_layer_launcher", lambda *a, **kw: launcher)
     monkeypatch.setattr(path, "_mark_decision", lambda event, dev: None)
+    monkeypatch.setattr(path, "_kept_sink_sums", lambda kv_cache, rows, heads: None)
     monkeypatch.setattr(path, "_decision_buffers",
                         lambda rows, dev: (torch.full((rows,), -1, dtype=torch.int64),
                                            torch.empty(rows, dtype=torch.int32), _Event()))

@@ -371,3 +371,148 @@ def test_stream_with_refresh_production_shape(gpu_device, heads, seed, calls):
         unit = max(1.0, want.abs().max().item())
         err = (got[:, idx.to(gpu_device)].float().cpu() - want).abs()
         assert err.max().item() <= 2e-2 * unit and err.mean().item() <= 2e-3 * unit, call
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("heads,ft_grid", [(3, GRID), (12, PROD_GRID)])
+def test_kept_frame_sums_give_the_same_bits(gpu_device, heads, ft_grid):
+    """With the sink frames' token sums kept between calls the operator reads
+    the new chunk only; similarities and decisions must be bit for bit those of
+    the call that sums every frame from the cache - through a sequence in which
+    frames go stale, a filling row lands in a sink frame and an evicting row
+    refreshes one."""
+    from streamdiffusionv2_amd import ops, rope
+
+    ft = ft_grid[1] * ft_grid[2]
+    rows, sink, frames = 2, 3, 5
+    gen = torch.Generator().manual_seed(77 + heads)
+    basis = torch.randn(3, heads * 128, generator=gen)
+    ck = torch.cat([directed_chunk(gen, rows, heads, torch.bfloat16, basis, ft=ft)[1] for _ in range(frames)], dim=1)
+    cv = torch.cat([directed_chunk(gen, rows, heads, torch.bfloat16, basis, ft=ft)[2] for _ in range(frames)], dim=1)
+    ck, cv = ck.to(gpu_device), cv.to(gpu_device)
+    table = ops.device_freqs(rope.build_freqs(), gpu_device)
+    kept = ops.new_sink_frame_sums(rows, heads, sink, gpu_device)
+    kept.fill_(float("nan"))                       # whatever it holds is stale
+    stale = [0b111, 0b111]
+
+    def both(k, v, starts, thr, planned, evicting):
+        override_a = torch.full((rows,), -5, dtype=torch.int64, device=gpu_device)
+        override_b = torch.full((rows,), -5, dtype=torch.int64, device=gpu_device)
+        sim_a, ref_a = ops.sink_similarity(k, v, ck, cv, table, ft_grid[1:], starts, sink, thr,
+                                           dst_start_override=override_a, override_rows=evicting)
+        sim_b, ref_b = ops.sink_similarity(k, v, ck, cv, table, ft_grid[1:], starts, sink, thr,
+                                           dst_start_override=override_b, override_rows=evicting,
+                                           frame_sums=kept, stale_frames=stale, planned_frames=planned)
+        torch.cuda.synchronize()
+        assert torch.equal(sim_a.view(torch.int32), sim_b.view(torch.int32))
+        assert ref_a.tolist() == ref_b.tolist() and override_a.tolist() == override_b.tolist()
+        return ref_b.tolist()
+
+    def chunk():
+        _, k, v = directed_chunk(gen, rows, heads, torch.bfloat16, basis, ft=ft)
+        return k.to(gpu_device), v.to(gpu_device)
+
+    # 1. everything stale, nothing lands in the sink
+    k, v = chunk()
+    both(k, v, [4, 9], THR, [-1, -1], [False, False])
+    stale = [0, 0]
+    # 2. nothing stale: only the new chunk is read (the cache rows of frame 1 of row 0 are scribbled over
+    #    behind the operator's back to show it: the kept sums still describe the old contents)
+    saved = ck[0, ft:2 * ft].clone()
+    ck[0, ft:2 * ft] = 0
+    k, v = chunk()
+    sim_kept, _ = ops.sink_similarity(k, v, ck, cv, table, ft_grid[1:], [5, 10], sink, THR, frame_sums=kept,
+                                      stale_frames=stale, planned_frames=[-1, -1])
+    ck[0, ft:2 * ft] = saved
+    sim_full, _ = ops.sink_similarity(k, v, ck, cv, table, ft_grid[1:], [5, 10], sink, THR)
+    torch.cuda.synchronize()
+    assert torch.equal(sim_kept.view(torch.int32), sim_full.view(torch.int32))
+    # 3. a filling row (row 1) lands in sink frame 2: the append is played by hand, the kept sums follow by themselves
+    k, v = chunk()
+    both(k, v, [6, 2], THR, [-1, 2], [False, False])
+    roped = ops.causal_rope_apply(k, [ft_grid] * rows, table, torch.tensor([6, 2]))
+    ck[1, 2 * ft:3 * ft] = roped[1]
+    cv[1, 2 * ft:3 * ft] = v[1]
+    k, v = chunk()
+    both(k, v, [7, 3], THR, [-1, -1], [False, False])
+    # 4. an evicting row (row 0) refreshes: threshold 1.5 always picks the minimum; the append follows the override
+    k, v = chunk()
+    chosen = both(k, v, [8, 4], 1.5, [-1, -1], [True, False])
+    assert chosen[0] >= 0
+    roped = ops.causal_rope_apply(k, [ft_grid] * rows, table, torch.tensor([8, 4]))
+    ck[0, chosen[0] * ft:(chosen[0] + 1) * ft] = roped[0]
+    cv[0, chosen[0] * ft:(chosen[0] + 1) * ft] = v[0]
+    k, v = chunk()
+    both(k, v, [9, 5], THR, [-1, -1], [False, False])
+    # 5. a frame written behind the operator's back and declared stale is summed again
+    ck[1, 0:ft] = ck[1, 3 * ft:4 * ft]
+    stale = [0, 0b001]
+    k, v = chunk()
+    both(k, v, [10, 6], THR, [-1, -1], [False, False])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("heads", [12, 40, 5])
+def test_similarity_with_the_key_norm_folded_in(gpu_device, heads):
+    """k handed over raw with its RMSNorm weight must give the bits of k
+    normalised beforehand by the oracle's WanRMSNorm."""
+    from streamdiffusionv2_amd import ops, rope
+
+    rows, sink, frames, eps = 2, 3, 4, 1e-6
+    gen = torch.Generator().manual_seed(500 + heads)
+    basis = torch.randn(3, heads * 128, generator=gen)
+    _, k_raw, v = directed_chunk(gen, rows, heads, torch.bfloat16, basis, scale=1.3)
+    weight = (torch.rand(heads * 128, generator=gen) + 0.5).bfloat16()
+    k_normed = oracle.wan_rms_norm(k_raw.flatten(2), weight, eps).view_as(k_raw)
+    ck = torch.cat([directed_chunk(gen, rows, heads, torch.bfloat16, basis)[1] for _ in range(frames)], dim=1)
+    cv = torch.cat([directed_chunk(gen, rows, heads, torch.bfloat16, basis)[2] for _ in range(frames)], dim=1)
+    table = ops.device_freqs(rope.build_freqs(), gpu_device)
+    args = (ck.to(gpu_device), cv.to(gpu_device), table, GRID[1:], [3, 8], sink, THR)
+    want, want_refresh = ops.sink_similarity(k_normed.to(gpu_device), v.to(gpu_device), *args)
+    got, got_refresh = ops.sink_similarity(k_raw.to(gpu_device), v.to(gpu_device), *args,
+                                           k_norm=(weight.to(gpu_device), eps))
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int32), want.view(torch.int32))
+    assert got_refresh.tolist() == want_refresh.tolist()
+
+
+@pytest.mark.gpu
+def test_module_with_fused_norm_and_adaptive_sink(gpu_device):
+    """The shipped combination: q / k norm inside the append AND the adaptive
+    sink check (which then normalises the new keys itself).  The stream must
+    leave the cache that the unfused module leaves (norms applied by torch on
+    the GPU add in another order: at most one ulp apart) and take the same
+    decisions."""
+    from streamdiffusionv2_amd import ring, rope
+    from streamdiffusionv2_amd.attention import CausalWanSelfAttention
+
+    torch.manual_seed(9)
+    dim, heads = 384, 3
+    mod = CausalWanSelfAttention(dim, heads).to(gpu_device).bfloat16()
+    with torch.no_grad():
+        mod.norm_q.weight.uniform_(0.5, 1.5)
+        mod.norm_k.weight.uniform_(0.5, 1.5)
+    mod.sink_size, mod.adapt_sink_thr = 2, 0.2
+    freqs = rope.build_freqs()
+    calls = 10
+    scenes = [torch.randn(1, 1, dim) * 2 for _ in range(3)]
+    xs = [(torch.randn(1, FT, dim) * 0.3 + scenes[c // 4]).bfloat16().to(gpu_device) for c in range(calls)]
+    runs = []
+    for fuse in (True, False):
+        mod.fuse_qk_norm = fuse
+        mod.evict_idx = None
+        cache = ring.new_kv_cache(1, 1, 5 * FT, heads, 1, device=gpu_device)[0]
+        decisions, outs = [], []
+        with torch.no_grad():
+            for c in range(calls):
+                outs.append(mod(xs[c], None, torch.tensor([GRID]), freqs, None, kv_cache=cache, current_start=c * FT))
+                decisions.append(mod.last_refresh)
+        runs.append((decisions, [list(q) for q in mod.evict_idx], cache["k"].clone(), cache["v"].clone(), torch.stack(outs)))
+    torch.cuda.synchronize()
+    (d1, q1, k1, v1, y1), (d0, q0, k0, v0, y0) = runs
+    assert d1 == d0 and q1 == q0
+    assert any(d is not None and d[0] >= 0 for d in d1)            # at least one refresh happened
+    assert torch.equal(v1, v0)
+    ik1, ik0 = k1.cpu().view(torch.int16).int(), k0.cpu().view(torch.int16).int()
+    assert (ik1 - ik0).abs().max().item() <= 1
+    assert (y1.float() - y0.float()).abs().max().item() <= 3e-2
