@@ -27,15 +27,90 @@ PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 
 
-# HBM bytes per launch at the default split counts, read with rocprofv3's
-# FETCH_SIZE and WRITE_SIZE counters (KiB per dispatch) on this same script and
-# scaled by what those counters read for a plain 256 MiB copy (x2.000 / x1.000).
-MEASURED_HBM_BYTES = {
-    "c2_wan1.3b_1560tok_6frames": {"attn": 85.54e6, "append": 29.09e6, "merge": 20.14e6, "splits": 3},
-    "c4_wan14b_1560tok_6frames": {"attn": 325.04e6, "append": 96.25e6, "merge": 84.02e6, "splits": 4},
-    "c3_wan1.3b_b4_4680tok_12frames": {"attn": 1071.13e6, "append": 345.47e6, "merge": 240.87e6, "splits": 3},
-    "c5_720p_b2_10800tok_21frames": {"attn": 3460.85e6, "append": 398.99e6, "merge": 566.36e6, "splits": 6},
-}
+# HBM bytes per launch, read with rocprofv3's FETCH_SIZE and WRITE_SIZE counters
+# (KiB per dispatch) on this same script and scaled by what those counters read
+# for the library's plain copy kernel: profiles/hbm_traffic.json, written by
+# `bench.py --record-traffic DIR` from the counter runs' CSV files.  A record is
+# only used for the kernels it was taken on: same key-range split count, same
+# kernel sources (hash below); otherwise `traffic` is null and stderr says why.
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+KERNEL_SOURCES = ("swa_attn_fwd.hip", "kv_append_rope.hip", "rope_device.h", "sdv2kv_internal.h")
+
+
+def kernel_source_hash() -> str:
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "streamdiffusionv2_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload_name: str, splits: int):
+    """The committed counter record for this workload, or None (with the reason on stderr)."""
+    try:
+        with open(TRAFFIC_JSON) as f:
+            rec = json.load(f)["workloads"].get(workload_name)
+    except (OSError, ValueError, KeyError) as e:
+        print(f"bench: no usable {TRAFFIC_JSON} ({e}): roofline.traffic is null", file=sys.stderr)
+        return None
+    if rec is None:
+        print(f"bench: {TRAFFIC_JSON} has no record for {workload_name}: roofline.traffic is null", file=sys.stderr)
+        return None
+    if rec["splits"] != splits or rec["kernel_sources"] != kernel_source_hash():
+        print(f"bench: the traffic record for {workload_name} was taken with {rec['splits']} key ranges on kernel "
+              f"sources {rec['kernel_sources']}, this run uses {splits} on {kernel_source_hash()}: counters must be "
+              "collected again (bench.py --record-traffic); roofline.traffic is null", file=sys.stderr)
+        return None
+    return rec
+
+
+def record_traffic(args, w):
+    """Turn the CSV files of four rocprofv3 counter runs under DIR (fetch/,
+    write/: this script on the workload; cfetch/, cwrite/: --calibrate-copy
+    256) into the workload's record in profiles/hbm_traffic.json."""
+    import collections
+    import csv
+    import glob
+
+    def per_kernel(sub):
+        files = glob.glob(os.path.join(args.record_traffic, sub, "**", "*counter_collection.csv"), recursive=True)
+        if not files:
+            raise SystemExit(f"no counter_collection.csv under {args.record_traffic}/{sub}")
+        total, count = collections.defaultdict(float), collections.Counter()
+        for row in csv.DictReader(open(files[0])):
+            for short in ("swa_attn_fwd_kernel", "kv_append_rope_kernel", "copy16_kernel"):
+                if short in row["Kernel_Name"]:
+                    total[short] += float(row["Counter_Value"])
+                    count[short] += 1
+        return {k: total[k] / count[k] for k in total}
+
+    fetch, write = per_kernel("fetch"), per_kernel("write")
+    cfetch, cwrite = per_kernel("cfetch"), per_kernel("cwrite")
+    copy_kib = 256 * 1024
+    f_scale, w_scale = copy_kib / cfetch["copy16_kernel"], copy_kib / cwrite["copy16_kernel"]
+    from streamdiffusionv2_amd import _capi
+
+    rec = {
+        "splits": args.num_splits or _capi.lib().sdv2_swa_attn_default_splits(w.rows, w.chunk_tokens, w.heads, w.cache_tokens),
+        "kernel_sources": kernel_source_hash(),
+        "fetch_scale": f_scale, "write_scale": w_scale,
+        "attn": (fetch["swa_attn_fwd_kernel"] * f_scale + write["swa_attn_fwd_kernel"] * w_scale) * 1024,
+        "append": (fetch["kv_append_rope_kernel"] * f_scale + write["kv_append_rope_kernel"] * w_scale) * 1024,
+        "attn_fetch_kib": fetch["swa_attn_fwd_kernel"], "attn_write_kib": write["swa_attn_fwd_kernel"],
+        "append_fetch_kib": fetch["kv_append_rope_kernel"], "append_write_kib": write["kv_append_rope_kernel"],
+    }
+    try:
+        with open(TRAFFIC_JSON) as f:
+            doc = json.load(f)
+    except (OSError, ValueError):
+        doc = {"unit": "bytes per launch (HBM reads + writes)", "workloads": {}}
+    doc["workloads"][w.name] = rec
+    with open(TRAFFIC_JSON, "w") as f:
+        json.dump(doc, f, indent=1, sort_keys=True)
+        f.write("\n")
+    print(json.dumps({w.name: rec}))
 
 
 def parse_args():
@@ -50,6 +125,9 @@ def parse_args():
     ap.add_argument("--cpu-layers", type=int, default=2)
     ap.add_argument("--calibrate-copy", type=int, default=0, metavar="MIB",
                     help="only run the library's plain copy kernel on MIB mebibytes (counter calibration)")
+    ap.add_argument("--record-traffic", metavar="DIR", default=None,
+                    help="no GPU work: read the counter CSVs of rocprofv3 runs under DIR (fetch/, write/, cfetch/, cwrite/) "
+                         "and write this workload's record into profiles/hbm_traffic.json")
     ap.add_argument("--fill-phase", action="store_true",
                     help="also time every chunk of a fresh stream while its ring fills (reported apart)")
     ap.add_argument("--qk-norm", action="store_true",
@@ -63,6 +141,9 @@ def parse_args():
                     help="also time the stream with the adaptive sink refresh on (one-frame chunks, one row)")
     ap.add_argument("--handoff", action="store_true",
                     help="also time the owner change of a layer's cache block (export to / import from the wire layout)")
+    ap.add_argument("--softmax-range", action="store_true",
+                    help="also time the attention launch with the queries scaled up until rows leave the range the fast "
+                         "softmax covers and waves redo their block with the running-maximum recurrence")
     ap.add_argument("--skip-mfma-reference", action="store_true",
                     help="do not time the vendor bf16 GEMM that shows what this box sustains on MFMA")
     return ap.parse_args()
@@ -237,7 +318,7 @@ def qk_norm_section(args, w):
     work done as the reference does it (two WanRMSNorm modules in torch, then
     the plain append kernel).  Times are per layer call, HIP events around a
     run of calls that rotates over all layers' tensors."""
-    from streamdiffusionv2_amd import ops, ring, workloads
+    from streamdiffusionv2_amd import _capi, ops, ring, workloads
     from streamdiffusionv2_amd.attention import WanRMSNorm
 
     dev = torch.device("cuda:0")
@@ -280,8 +361,50 @@ def qk_norm_section(args, w):
         torch.cuda.synchronize()
         out[name] = e0.elapsed_time(e1) / n
     out["bytes_per_launch"] = w.append_bytes(with_q=True)
-    out["fused_GBps"] = out["bytes_per_launch"] / (out["fused_ms"] * 1e-3) / 1e9
-    out["note"] = "host-inclusive per-call times; the torch path launches about a dozen kernels per call"
+    # the fused kernel's own duration (timing events in its dispatch)
+    timer = ops.KernelTimer()
+    kernel_ms = []
+    for i in range(n):
+        timer.arm(_capi.KERNEL_APPEND)
+        fused(i)
+        kernel_ms.append(timer.elapsed_ms())
+    timer.close()
+    out["fused_kernel_ms"] = sum(kernel_ms) / len(kernel_ms)
+    out["fused_kernel_GBps"] = out["bytes_per_launch"] / (out["fused_kernel_ms"] * 1e-3) / 1e9
+    out["note"] = ("fused_ms / torch_norms_plus_append_ms are host-inclusive per-call times (the torch path launches "
+                   "about a dozen kernels per call); fused_kernel_ms is the kernel alone")
+    # The consumer side (causal_model.py:387-389): the o projection reads the attention output in place.
+    # Per layer: attention alone, the vendor GEMM alone, and the two back to back on one stream.
+    dim = H * 128
+    w_o = (torch.randn(dim, dim, device=dev) * dim ** -0.5).to(w.dtype)
+    kc = [c["k"] for c in caches]
+    vc = [c["v"] for c in caches]
+    for c in caches:
+        c["k"].normal_()
+        c["v"].normal_()
+    attn_out = torch.empty_like(qkv[0][0])
+
+    def attention(i):
+        ops.swa_attention(qkv[i % layers][0], kc[i % layers], vc[i % layers], None, out=attn_out)
+
+    def o_proj(i):
+        torch.nn.functional.linear(attn_out.flatten(2), w_o)
+
+    def both(i):
+        attention(i)
+        o_proj(i)
+
+    for name, fn in (("attention_ms", attention), ("o_proj_gemm_ms", o_proj), ("attention_then_o_proj_ms", both)):
+        for i in range(layers):
+            fn(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(n):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        out[name] = e0.elapsed_time(e1) / n
     return out
 
 
@@ -443,6 +566,52 @@ def handoff_section(args, w):
     return out
 
 
+def softmax_range_section(args, w):
+    """What leaving the fast softmax's range costs.  The kernel takes exp2 of
+    every scaled score against a fixed per-row reference (the largest score
+    among the first 32 keys of the workgroup's range); a row whose later scores
+    exceed that reference by about 100 in log2 units overflows, and the wave
+    that holds it redoes its 32-row block with the running-maximum recurrence
+    while the other waves of the workgroup keep the tiles coming.  Here the
+    queries are scaled by growing factors (scores of standard deviation
+    factor * chunk scale^2 * sqrt(128) in natural units), and then ONE query row
+    alone is made extreme."""
+    from streamdiffusionv2_amd import ops
+
+    dev = torch.device("cuda:0")
+    B, S, H, L = w.rows, w.chunk_tokens, w.heads, w.cache_tokens
+    gen = torch.Generator(device=dev).manual_seed(3)
+    q = torch.randn(B, S, H, 128, device=dev, generator=gen)
+    k = torch.randn(B, H, L, 128, device=dev, generator=gen).bfloat16().permute(0, 2, 1, 3)
+    v = torch.randn(B, H, L, 128, device=dev, generator=gen).bfloat16().permute(0, 2, 1, 3)
+    out = torch.empty(B, S, H, 128, device=dev, dtype=torch.bfloat16)
+
+    def timed(qq, iters=20):
+        qq = qq.bfloat16()
+        for _ in range(3):
+            ops.swa_attention(qq, k, v, None, out=out)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(iters):
+            ops.swa_attention(qq, k, v, None, out=out)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters
+
+    res = {"score_std_nat_at_factor_1": float((128 ** 0.5) / (128 ** 0.5)), "factors": {}}
+    plain = timed(q)
+    res["plain_ms"] = plain
+    for factor in (4, 16, 32, 64, 128, 256):
+        ms = timed(q * factor)
+        res["factors"][str(factor)] = {"ms": ms, "ratio_to_plain": ms / plain, "finite": bool(torch.isfinite(out.float()).all())}
+    one = q.clone()
+    one[0, S // 2, :, :] *= 300.0
+    ms = timed(one)
+    res["one_extreme_row_of_%d" % S] = {"ms": ms, "ratio_to_plain": ms / plain, "finite": bool(torch.isfinite(out.float()).all())}
+    return res
+
+
 def cpu_baseline(args, w):
     """The CPU oracle (a PyTorch restatement of the reference's op sequence)
     on this box's host cores: a bounded sample of steady-state chunks on a few
@@ -505,6 +674,9 @@ def main():
         print("the GPU attention kernel computes in bf16; workload 1 is the CPU-plumbing parity case, "
               "not a bench line", file=sys.stderr)
         sys.exit(2)
+    if args.record_traffic:
+        record_traffic(args, w)
+        return
     if not torch.cuda.is_available():
         print("bench.py needs a GPU (the KV-cache path has no CPU fallback)", file=sys.stderr)
         sys.exit(2)
@@ -529,9 +701,7 @@ def main():
     achieved_tflops = w.attn_flops() / attn_s / 1e12
     # the query is rotated inside the attention kernel: the append moves K and V only
     append_gbs = w.append_bytes(with_q=False) / (g["append_ms"] * 1e-3) / 1e9
-    hbm = MEASURED_HBM_BYTES.get(w.name)
-    if hbm is not None and hbm["splits"] != g["splits"]:
-        hbm = None
+    hbm = measured_traffic(w.name, g["splits"])
     result = {
         "metric": "kv_append_attn_tokens_per_s",
         "value": tokens / (g["ms_per_step"] * 1e-3),
@@ -584,6 +754,8 @@ def main():
         result["handoff"] = handoff_section(args, w)
     if args.adaptive_sink:
         result["adaptive_sink"] = adaptive_sink_section(args, w)
+    if args.softmax_range:
+        result["softmax_range"] = softmax_range_section(args, w)
     if args.torch_reference:
         result["torch_gpu_reference"] = torch_reference_section(args, w, g["ms_per_step"])
     if not args.skip_mfma_reference:

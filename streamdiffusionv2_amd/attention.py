@@ -10,6 +10,7 @@ two HIP kernels and no device-to-host copy.
 """
 from __future__ import annotations
 
+import copy
 from typing import List, Optional
 
 import torch
@@ -262,81 +263,91 @@ class RingKVPath:
             else:
                 queues_before = [list(queue) for queue in self._evict_idx]
 
-        # planned as if no row refreshed; _settle() corrects the host state later where one did
-        plan = ring.plan_append(kv_cache, self._evict_idx, starts, q.shape[1], frame_tokens, self.sink_size)
-        override = None
-        if adaptive:
-            # adaptive sink refresh (causal_model.py:284-299): one fused
-            # reduction on the device, whose decision goes straight to the
-            # append below and, written into pinned memory by the kernel, to the host
-            override, host, event = self._decision_buffers(rows, q.device)
-            kept = self._kept_sink_sums(kv_cache, rows, q.shape[2])
-            extra = {}
-            if kept is not None:
-                # where the chunk lands by the plan, if that is a sink frame: a row still filling,
-                # or an evicting one whose queue is headed by a refresh decided while it was filling
-                planned = [d // frame_tokens if d < self.sink_size * frame_tokens else -1 for d in plan.dst_start]
-                extra = dict(frame_sums=kept["sums"], stale_frames=list(kept["stale"]), planned_frames=planned)
-                kept["stale"] = [0] * rows        # summed now, and kept current by the decision kernel from here on
-            ops.sink_similarity(
-                k, v, kv_cache["k"], kv_cache["v"], table, (h, w), [c // frame_tokens for c in starts],
-                self.sink_size, self.adapt_sink_thr, dst_start_override=override, override_rows=plan.evicting,
-                refresh_out=host, k_norm=k_norm, **extra)
-            self._mark_decision(event, q.device)
-            self._pending = dict(event=event, host=host, plan=plan, queues=queues_before, starts=list(starts),
-                                 tokens=q.shape[1], frame_tokens=frame_tokens, sink_size=self.sink_size,
-                                 cap=kv_cache["k"].shape[1])
-        if not adaptive:
-            self._sink_frames_written(kv_cache, plan, q.shape[1], frame_tokens)
-        span = plan.max_seq_len
-        seq = None
-        if any(n != span for n in plan.new_local_end):
-            # rows differ only while the stream batch is still filling; the
-            # lengths are a handful of host ints, shipped asynchronously
-            seq = torch.tensor(plan.new_local_end, dtype=torch.int32).to(q.device, non_blocking=True)
-        self._last_plan = plan
-        mask_tokens = 0
-        if self.block_frames is not None and self.block_frames * frame_tokens < q.shape[1]:
-            mask_tokens = self.block_frames * frame_tokens
+        # Planning advances the host's ring state (queues, pass counter, index mirror) before the launches
+        # are validated: a call that fails - a frame beyond the RoPE table, say - must leave it where it was.
+        undo = (copy.deepcopy(self._evict_idx), kv_cache.get("current_step"))
+        try:
+            # planned as if no row refreshed; _settle() corrects the host state later where one did
+            plan = ring.plan_append(kv_cache, self._evict_idx, starts, q.shape[1], frame_tokens, self.sink_size)
+            override = None
+            if adaptive:
+                # adaptive sink refresh (causal_model.py:284-299): one fused
+                # reduction on the device, whose decision goes straight to the
+                # append below and, written into pinned memory by the kernel, to the host
+                override, host, event = self._decision_buffers(rows, q.device)
+                kept = self._kept_sink_sums(kv_cache, rows, q.shape[2])
+                extra = {}
+                if kept is not None:
+                    # where the chunk lands by the plan, if that is a sink frame: a row still filling,
+                    # or an evicting one whose queue is headed by a refresh decided while it was filling
+                    planned = [d // frame_tokens if d < self.sink_size * frame_tokens else -1 for d in plan.dst_start]
+                    extra = dict(frame_sums=kept["sums"], stale_frames=list(kept["stale"]), planned_frames=planned)
+                    kept["stale"] = [0] * rows        # summed now, and kept current by the decision kernel from here on
+                ops.sink_similarity(
+                    k, v, kv_cache["k"], kv_cache["v"], table, (h, w), [c // frame_tokens for c in starts],
+                    self.sink_size, self.adapt_sink_thr, dst_start_override=override, override_rows=plan.evicting,
+                    refresh_out=host, k_norm=k_norm, **extra)
+                self._mark_decision(event, q.device)
+                self._pending = dict(event=event, host=host, plan=plan, queues=queues_before, starts=list(starts),
+                                     tokens=q.shape[1], frame_tokens=frame_tokens, sink_size=self.sink_size,
+                                     cap=kv_cache["k"].shape[1])
+            if not adaptive:
+                self._sink_frames_written(kv_cache, plan, q.shape[1], frame_tokens)
+            span = plan.max_seq_len
+            seq = None
+            if any(n != span for n in plan.new_local_end):
+                # rows differ only while the stream batch is still filling; the
+                # lengths are a handful of host ints, shipped asynchronously
+                seq = torch.tensor(plan.new_local_end, dtype=torch.int32).to(q.device, non_blocking=True)
+            self._last_plan = plan
+            mask_tokens = 0
+            if self.block_frames is not None and self.block_frames * frame_tokens < q.shape[1]:
+                mask_tokens = self.block_frames * frame_tokens
 
-        if q.dtype == torch.bfloat16 and rows <= ops._capi.MAX_ROWS:
-            # steady-state fast path: launch descriptors are built once per
-            # (cache, shape) and only patched per call
-            launcher = self._layer_launcher(q, k, v, kv_cache, table, (f, h, w), qk_norm)
-            start_frames = [c // frame_tokens for c in starts]
-            out = launcher.launch(q, k, v, start_frames, plan, seq, mask_tokens, override)
+            if q.dtype == torch.bfloat16 and rows <= ops._capi.MAX_ROWS:
+                # steady-state fast path: launch descriptors are built once per
+                # (cache, shape) and only patched per call
+                launcher = self._layer_launcher(q, k, v, kv_cache, table, (f, h, w), qk_norm)
+                start_frames = [c // frame_tokens for c in starts]
+                out = launcher.launch(q, k, v, start_frames, plan, seq, mask_tokens, override)
+                if return_roped_query:
+                    # the attention kernel rotates q on the fly and keeps no copy: the
+                    # stand-alone rotation gives the same bits (one arithmetic for both)
+                    if launcher.roped_q is not None:
+                        return out, launcher.roped_q.clone()
+                    return out, ops.causal_rope_apply(q, [(f, h, w)] * rows, table, torch.tensor(start_frames))
+                return out
+
+            roped_q = ops.kv_append_rope(
+                q, k, v, kv_cache["k"], kv_cache["v"], table, (f, h, w),
+                [c // frame_tokens for c in starts], plan.dst_start,
+                global_end_index=kv_cache["global_end_index"],
+                local_end_index=kv_cache["local_end_index"],
+                new_global_end=plan.new_global_end,
+                new_local_end=plan.new_local_end,
+                qk_norm=qk_norm,
+                dst_start_override=override,
+            )
+            mask = dict(chunk_key_start=list(plan.dst_start), mask_block_tokens=mask_tokens) if mask_tokens else {}
+            if roped_q.dtype == torch.bfloat16:
+                out = ops.swa_attention(roped_q, kv_cache["k"][:, :span], kv_cache["v"][:, :span], seq, **mask)
+            else:
+                # fp32 storage is a plumbing mode (the reference's CPU-runnable
+                # configuration): RoPE, cache and indices stay fp32 and bit-exact,
+                # the attention kernel computes in bf16 on down-cast copies.
+                out = ops.swa_attention(
+                    roped_q.bfloat16(), kv_cache["k"][:, :span].bfloat16(), kv_cache["v"][:, :span].bfloat16(), seq, **mask
+                ).to(roped_q.dtype)
             if return_roped_query:
-                # the attention kernel rotates q on the fly and keeps no copy: the
-                # stand-alone rotation gives the same bits (one arithmetic for both)
-                if launcher.roped_q is not None:
-                    return out, launcher.roped_q.clone()
-                return out, ops.causal_rope_apply(q, [(f, h, w)] * rows, table, torch.tensor(start_frames))
+                return out, roped_q
             return out
 
-        roped_q = ops.kv_append_rope(
-            q, k, v, kv_cache["k"], kv_cache["v"], table, (f, h, w),
-            [c // frame_tokens for c in starts], plan.dst_start,
-            global_end_index=kv_cache["global_end_index"],
-            local_end_index=kv_cache["local_end_index"],
-            new_global_end=plan.new_global_end,
-            new_local_end=plan.new_local_end,
-            qk_norm=qk_norm,
-            dst_start_override=override,
-        )
-        mask = dict(chunk_key_start=list(plan.dst_start), mask_block_tokens=mask_tokens) if mask_tokens else {}
-        if roped_q.dtype == torch.bfloat16:
-            out = ops.swa_attention(roped_q, kv_cache["k"][:, :span], kv_cache["v"][:, :span], seq, **mask)
-        else:
-            # fp32 storage is a plumbing mode (the reference's CPU-runnable
-            # configuration): RoPE, cache and indices stay fp32 and bit-exact,
-            # the attention kernel computes in bf16 on down-cast copies.
-            out = ops.swa_attention(
-                roped_q.bfloat16(), kv_cache["k"][:, :span].bfloat16(), kv_cache["v"][:, :span].bfloat16(), seq, **mask
-            ).to(roped_q.dtype)
-        if return_roped_query:
-            return out, roped_q
-        return out
-
+        except Exception:
+            self._evict_idx, self._pending, self._sink_sums = undo[0], None, None
+            if undo[1] is not None:
+                kv_cache["current_step"] = undo[1]
+            ring.forget_index_mirror(kv_cache)        # the device tensors are authoritative again
+            raise
 
 class CausalWanSelfAttention(nn.Module, RingKVPath):
 

@@ -207,3 +207,48 @@ def test_fused_norm_argument_errors(gpu_device):
         ops.kv_append_rope(x, x, x, cache, cache.clone(), table, (1, 2, 3), [0], [0], qk_norm=(w.float(), w, 1e-6))
     with pytest.raises(RuntimeError):       # k only
         ops.kv_append_rope(None, x, x, cache, cache.clone(), table, (1, 2, 3), [0], [0], qk_norm=(w, w, 1e-6))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fuse", [True, False])
+def test_output_projection_reads_the_kernels_output_in_place(gpu_device, fuse):
+    """The o projection (causal_model.py:387-389, x.flatten(2) -> self.o) must
+    consume the tensor the attention kernel wrote: same storage, contiguous
+    [B, S, heads * 128], nothing copied or re-laid-out in between.  And on the
+    way in, with the norm folded into the append, the q / k projections' raw
+    outputs reach the kernel as views of what the GEMMs wrote."""
+    from streamdiffusionv2_amd import ring, rope
+    from streamdiffusionv2_amd.attention import CausalWanSelfAttention
+
+    torch.manual_seed(4)
+    dim, heads, grid = 256, 2, (1, 4, 6)
+    S = 24
+    mod = CausalWanSelfAttention(dim, heads).to(gpu_device).bfloat16()
+    mod.sink_size, mod.fuse_qk_norm = 1, fuse
+    seen = {}
+    inner_attend = mod.attend
+
+    def spying_attend(q, k, v, *args, **kw):
+        seen["q_in"], seen["k_in"] = q, k
+        out = inner_attend(q, k, v, *args, **kw)
+        seen["attn_out"] = out
+        return out
+
+    mod.attend = spying_attend
+    proj_out = {}
+    for name in ("q", "k"):
+        getattr(mod, name).register_forward_hook(lambda m, i, o, name=name: proj_out.__setitem__(name, o))
+    mod.o.register_forward_pre_hook(lambda m, inputs: seen.__setitem__("o_in", inputs[0]))
+    cache = ring.new_kv_cache(1, 1, 3 * S, heads, 1, device=gpu_device)[0]
+    x = torch.randn(1, S, dim, device=gpu_device).bfloat16()
+    with torch.no_grad():
+        y = mod(x, None, torch.tensor([grid]), rope.build_freqs(), None, kv_cache=cache, current_start=0)
+    torch.cuda.synchronize()
+    o_in, attn_out = seen["o_in"], seen["attn_out"]
+    assert o_in.data_ptr() == attn_out.data_ptr()
+    assert o_in.is_contiguous() and tuple(o_in.shape) == (1, S, dim)
+    assert attn_out.is_contiguous() and tuple(attn_out.shape) == (1, S, heads, 128)
+    assert tuple(y.shape) == (1, S, dim)
+    if fuse:
+        assert seen["q_in"].data_ptr() == proj_out["q"].data_ptr()
+        assert seen["k_in"].data_ptr() == proj_out["k"].data_ptr()

@@ -263,3 +263,45 @@ def test_one_workspace_serves_changing_shapes(gpu_device):
             assert torch.equal(got, first[key])
         first[key] = got
         assert not ws[:65536].any()                     # the ticket words
+
+
+def test_one_extreme_query_row_costs_less_than_a_second_launch(gpu_device):
+    """A single query row whose scores leave the fast softmax's range sends one
+    wave of one workgroup through the running-maximum pass, not the whole
+    launch: the result stays right for that row and its neighbours, and the
+    launch stays under twice the time of the plain one (Wan 1.3B shape: 1560
+    queries against six frames, 12 heads)."""
+    from streamdiffusionv2_amd import ops
+
+    gen = torch.Generator(device=gpu_device).manual_seed(21)
+    S, H, L = 1560, 12, 9360
+    q = torch.randn(1, S, H, 128, device=gpu_device, generator=gen)
+    k = torch.randn(1, H, L, 128, device=gpu_device, generator=gen).bfloat16().permute(0, 2, 1, 3)
+    v = torch.randn(1, H, L, 128, device=gpu_device, generator=gen).bfloat16().permute(0, 2, 1, 3)
+    hot = q.clone()
+    hot[0, 777] *= 300.0                    # scores of some thousand nats: far outside +-69 around any reference
+    out = torch.empty(1, S, H, 128, device=gpu_device, dtype=torch.bfloat16)
+
+    def timed(qq):
+        qq = qq.bfloat16()
+        for _ in range(3):
+            ops.swa_attention(qq, k, v, None, out=out)
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(7):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(5):
+                ops.swa_attention(qq, k, v, None, out=out)
+            e1.record()
+            torch.cuda.synchronize()
+            times.append(e0.elapsed_time(e1) / 5)
+        return sorted(times)[3]
+
+    plain = timed(q)
+    extreme = timed(hot)
+    rows = torch.tensor([0, 776, 777, 778, 1559])
+    want = oracle.attention_fp32_reference(hot.bfloat16().cpu()[:, rows], k.cpu(), v.cpu(), [L])
+    _check(out.cpu()[:, rows], want)
+    print(f"plain {plain * 1e3:.1f} us, one extreme row {extreme * 1e3:.1f} us", flush=True)
+    assert extreme < 2.0 * plain, (plain, extreme)

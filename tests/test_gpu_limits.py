@@ -80,3 +80,40 @@ def test_stream_path_on_either_side_of_the_row_limit(gpu_device, rows):
         want = oracle.attention_fp32_reference(want_q, o_cache["k"], o_cache["v"], seq)
         err = (got.float().cpu() - want).abs()
         assert err.max().item() <= 2e-2 and err.mean().item() <= 2e-3
+
+
+@pytest.mark.gpu
+def test_a_failed_call_leaves_the_ring_state_where_it_was(gpu_device):
+    """Planning advances the host's ring state before the launch is validated;
+    a call the library refuses (here: a frame beyond the 1024 rows of the RoPE
+    table) must not leave queue, pass counter or index mirror advanced while
+    the device indices stayed put - the stream continues as if it had not been made."""
+    import copy
+
+    from streamdiffusionv2_amd import ring, rope
+    from streamdiffusionv2_amd.attention import RingKVPath
+
+    torch.manual_seed(0)
+    heads, grid, S = 2, (1, 4, 6), 24
+    freqs = rope.build_freqs()
+    cache = ring.new_kv_cache(1, 1, 4 * S, heads, 1, device=gpu_device)[0]
+    twin = ring.new_kv_cache(1, 1, 4 * S, heads, 1, device=gpu_device)[0]
+    path, twin_path = RingKVPath(sink_size=1), RingKVPath(sink_size=1)
+    chunks = [tuple(torch.randn(1, S, heads, 128, device=gpu_device).bfloat16() for _ in range(3)) for _ in range(7)]
+    for c in range(5):
+        path.attend(*chunks[c], torch.tensor([grid]), freqs, cache, [c * S])
+        twin_path.attend(*chunks[c], torch.tensor([grid]), freqs, twin, [c * S])
+    before = (copy.deepcopy(path.evict_idx), cache["current_step"], cache["global_end_index"].tolist(),
+              cache["local_end_index"].tolist(), cache["k"].clone())
+    with pytest.raises(RuntimeError):
+        path.attend(*chunks[5], torch.tensor([grid]), freqs, cache, [2000 * S])      # frame 2000: beyond the table
+    torch.cuda.synchronize()
+    assert path.evict_idx == before[0] and cache["current_step"] == before[1]
+    assert cache["global_end_index"].tolist() == before[2] and cache["local_end_index"].tolist() == before[3]
+    assert torch.equal(cache["k"], before[4])
+    for c in (5, 6):
+        a = path.attend(*chunks[c], torch.tensor([grid]), freqs, cache, [c * S])
+        b = twin_path.attend(*chunks[c], torch.tensor([grid]), freqs, twin, [c * S])
+        assert torch.equal(a, b)
+    assert path.evict_idx == twin_path.evict_idx
+    assert torch.equal(cache["k"], twin["k"]) and torch.equal(cache["v"], twin["v"])
