@@ -141,6 +141,9 @@ def parse_args():
                     help="also time the stream with the adaptive sink refresh on (one-frame chunks, one row)")
     ap.add_argument("--handoff", action="store_true",
                     help="also time the owner change of a layer's cache block (export to / import from the wire layout)")
+    ap.add_argument("--launch-floor", action="store_true",
+                    help="also time the library's plain copy kernel on 16 bytes (what any launch costs) and on the "
+                         "append's byte count (what a pure stream of that size costs): the floor under the append kernel")
     ap.add_argument("--softmax-range", action="store_true",
                     help="also time the attention launch with the queries scaled up until rows leave the range the fast "
                          "softmax covers and waves redo their block with the running-maximum recurrence")
@@ -566,6 +569,36 @@ def handoff_section(args, w):
     return out
 
 
+def launch_floor_section(args, w):
+    """Kernel durations (timing events in the dispatch) of the library's plain
+    16-byte-vector copy kernel: on 16 bytes - a launch that does nothing - and
+    on as many bytes as the append kernel moves for this workload.  The append
+    cannot be faster than the first and has no reason to be faster than the
+    second; both are quoted beside it."""
+    from streamdiffusionv2_amd import _capi, ops
+
+    dev = torch.device("cuda:0")
+    out = {}
+    timer = ops.KernelTimer()
+    lib = _capi.lib()
+    moved = w.append_bytes(with_q=False)
+    for name, nbytes in (("empty_launch_us", 16), ("copy_of_append_bytes_us", moved // 2 // 16 * 16)):
+        src = torch.empty(nbytes, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        times = []
+        for i in range(60):
+            _capi.check(lib.sdv2_profile_time_next(_capi.KERNEL_COPY, timer.start, timer.stop), "time_next")
+            ops.copy_bytes(dst, src)
+            if i >= 10:
+                times.append(timer.elapsed_ms() * 1e3)
+        times.sort()
+        out[name] = times[len(times) // 2]
+    out["append_bytes"] = moved
+    out["copy_GBps"] = moved / (out["copy_of_append_bytes_us"] * 1e-6) / 1e9
+    timer.close()
+    return out
+
+
 def softmax_range_section(args, w):
     """What leaving the fast softmax's range costs.  The kernel takes exp2 of
     every scaled score against a fixed per-row reference (the largest score
@@ -754,6 +787,8 @@ def main():
         result["handoff"] = handoff_section(args, w)
     if args.adaptive_sink:
         result["adaptive_sink"] = adaptive_sink_section(args, w)
+    if args.launch_floor:
+        result["launch_floor"] = launch_floor_section(args, w)
     if args.softmax_range:
         result["softmax_range"] = softmax_range_section(args, w)
     if args.torch_reference:

@@ -22,7 +22,8 @@ typedef enum sdv2_profile_kernel {
   SDV2_KERNEL_RELAYOUT = 2,    /* sdv2_cache_relayout                          */
   SDV2_KERNEL_SINK_SUM = 3,    /* sdv2_sink_similarity: frame sums             */
   SDV2_KERNEL_SINK_DECIDE = 4, /* sdv2_sink_similarity: decision               */
-  SDV2_KERNEL_COUNT = 5
+  SDV2_KERNEL_COPY = 5,        /* sdv2_copy_bytes                              */
+  SDV2_KERNEL_COUNT = 6
 } sdv2_profile_kernel;
 
 /* ------------------------------------------------------------------------

@@ -28,7 +28,7 @@ STATIC_SCRATCH_BYTES = 64 << 20
 DTYPE_BF16 = 0
 DTYPE_F32 = 1
 
-KERNEL_APPEND, KERNEL_ATTENTION, KERNEL_RELAYOUT, KERNEL_SINK_SUM, KERNEL_SINK_DECIDE = range(5)
+KERNEL_APPEND, KERNEL_ATTENTION, KERNEL_RELAYOUT, KERNEL_SINK_SUM, KERNEL_SINK_DECIDE, KERNEL_COPY = range(6)
 
 # every symbol include/sdv2kv.h and include/sdv2kv_profile.h declare
 EXPORTED_SYMBOLS = (

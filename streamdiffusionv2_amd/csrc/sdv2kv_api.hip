@@ -11,9 +11,15 @@ namespace {
 
 thread_local sdv2::TimingPair armed[SDV2_KERNEL_COUNT];
 
-__global__ __launch_bounds__(256) void copy16_kernel(uint4* dst, const uint4* src, size_t n16) {
+struct CopyArgs {
+  uint4* dst;
+  const uint4* src;
+  size_t n16;
+};
+
+__global__ __launch_bounds__(256) void copy16_kernel(const CopyArgs a) {
   const size_t stride = (size_t)gridDim.x * blockDim.x;
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < a.n16; i += stride) a.dst[i] = a.src[i];
 }
 
 }  // namespace
@@ -75,7 +81,8 @@ extern "C" int sdv2_copy_bytes(void* dst, const void* src, size_t bytes, void* s
   const size_t n16 = bytes / 16;
   size_t blocks = (n16 + 255) / 256;
   if (blocks > 256 * 32) blocks = 256 * 32;
-  hipLaunchKernelGGL(copy16_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
-                     static_cast<uint4*>(dst), static_cast<const uint4*>(src), n16);
+  const CopyArgs args{static_cast<uint4*>(dst), static_cast<const uint4*>(src), n16};
+  sdv2::launch_timed(SDV2_KERNEL_COPY, copy16_kernel, dim3((unsigned)blocks), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), args);
   return hipGetLastError() == hipSuccess ? SDV2_OK : SDV2_ERR_LAUNCH;
 }
