@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SDV2KV_ABI_VERSION 8
+#define SDV2KV_ABI_VERSION 9
 #define SDV2_HEAD_DIM 128      /* causal_stream_inference.py:99-100 fixes 128 */
 #define SDV2_MAX_ROWS 16       /* rows (B) per sdv2_kv_append_rope call       */
 #define SDV2_MAX_SINK_FRAMES 16 /* sink frames per sdv2_sink_similarity call  */
@@ -258,7 +258,10 @@ typedef struct sdv2_sink_sim_params {
   const int64_t* start_frame;  /* host [B]: current_start // tokens            */
   float* similarity;           /* device float [B, sink_frames]                */
   int32_t* refresh;            /* device int32 [B]                             */
-  void* workspace;             /* device scratch for the frame means           */
+  void* workspace;             /* device scratch, sdv2_sink_similarity_workspace_bytes():
+                                * its first 256 bytes are ticket words that must be ZERO
+                                * when the buffer is first used (every call leaves them at
+                                * zero); calls that overlap in time need a buffer each      */
   size_t workspace_bytes;
   void* stream;                /* hipStream_t                                  */
   /* Optional hand-over to the append that follows on the stream: device int64
@@ -275,17 +278,17 @@ typedef struct sdv2_sink_sim_params {
    * the weight (heads * 128 elements of the tensors' dtype) and eps.          */
   const void* k_norm_weight;
   float norm_eps;
-  /* Optional: token sums of the cached sink frames kept between calls
-   * (device, sdv2_sink_frame_sums_bytes(), any initial contents).  The sums of
-   * a sink frame only change when the frame is written, so a caller that
-   * brings this buffer has the call read the new chunk alone:
+  /* Optional: the means of the cached sink frames kept between calls (device,
+   * sdv2_sink_frame_sums_bytes(), any initial contents, opaque to the caller).
+   * The mean of a sink frame only changes when the frame is written, so a
+   * caller that brings this buffer has the call read the new chunk alone:
    *   - stale_frames[i] (host [B]): bit j set = sink frame j of row i was
    *     written by something other than the appends this call was told about
-   *     since its sums were last taken (or never summed): it is summed from the
+   *     since its mean was last taken (or never summed): it is summed from the
    *     cache in this call;
    *   - planned_frame[i] (host [B]): the sink frame the append that follows
    *     writes row i's chunk to by the caller's plan (a cache still filling,
-   *     or a queue headed by an earlier refresh), or -1.  The new chunk's sums
+   *     or a queue headed by an earlier refresh), or -1.  The new chunk's means
    *     are then filed as that frame's; for a row flagged in override_rows
    *     that refreshes in this call, as the refreshed frame's instead.
    * All three NULL: every sink frame is summed from the cache, every call.    */

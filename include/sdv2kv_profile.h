@@ -20,10 +20,9 @@ typedef enum sdv2_profile_kernel {
   SDV2_KERNEL_APPEND = 0,      /* sdv2_kv_append_rope                          */
   SDV2_KERNEL_ATTENTION = 1,   /* sdv2_swa_attn_fwd                            */
   SDV2_KERNEL_RELAYOUT = 2,    /* sdv2_cache_relayout                          */
-  SDV2_KERNEL_SINK_SUM = 3,    /* sdv2_sink_similarity: frame sums             */
-  SDV2_KERNEL_SINK_DECIDE = 4, /* sdv2_sink_similarity: decision               */
-  SDV2_KERNEL_COPY = 5,        /* sdv2_copy_bytes                              */
-  SDV2_KERNEL_COUNT = 6
+  SDV2_KERNEL_SINK = 3,        /* sdv2_sink_similarity                         */
+  SDV2_KERNEL_COPY = 4,        /* sdv2_copy_bytes                              */
+  SDV2_KERNEL_COUNT = 5
 } sdv2_profile_kernel;
 
 /* ------------------------------------------------------------------------

@@ -12,7 +12,7 @@ from typing import Optional
 
 LIB_PATH = Path(__file__).resolve().parent / "_lib" / "libsdv2kv.so"
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 HEAD_DIM = 128
 MAX_ROWS = 16
 
@@ -28,7 +28,7 @@ STATIC_SCRATCH_BYTES = 64 << 20
 DTYPE_BF16 = 0
 DTYPE_F32 = 1
 
-KERNEL_APPEND, KERNEL_ATTENTION, KERNEL_RELAYOUT, KERNEL_SINK_SUM, KERNEL_SINK_DECIDE, KERNEL_COPY = range(6)
+KERNEL_APPEND, KERNEL_ATTENTION, KERNEL_RELAYOUT, KERNEL_SINK, KERNEL_COPY = range(5)
 
 # every symbol include/sdv2kv.h and include/sdv2kv_profile.h declare
 EXPORTED_SYMBOLS = (

@@ -6,25 +6,25 @@
 // incoming one-frame chunk's roped K and its V; the two similarities are
 // averaged and, when the smallest falls below the threshold, that sink frame
 // is to be overwritten next.  The reference does this with four reductions and
-// two host round trips per row; here one reduction kernel sums every frame
-// over its tokens, eight token ranges per (frame, head) side by side (rotating
-// the new keys on the fly with the append kernel's arithmetic, so they never
-// have to be staged), and a second, tiny kernel turns the sums into means,
-// similarities and the decision.  The caller reads back one int per row
-// - not necessarily at once: the decision kernel can also hand the slot a
-// refresh selects straight to the append kernel that follows it on the stream
-// (dst_start_override), so the host may pick the decision up a whole model
-// pass later, when it plans this layer's next call.
+// two host round trips per row; here ONE launch does it: workgroups sum the
+// frames over their tokens, eight token ranges per (frame, head) side by side
+// (rotating the new keys on the fly with the append kernel's arithmetic, so
+// they never have to be staged), and the workgroup that finishes last for a
+// row turns the sums into means, similarities and the decision.  The caller
+// reads back one int per row - not necessarily at once: the decision can also
+// hand the slot a refresh selects straight to the append kernel that follows
+// on the stream (dst_start_override), so the host may pick the decision up a
+// whole model pass later, when it plans this layer's next call.
 //
 // Rounding follows the storage dtype: with bf16 tensors the frame means, the
 // two cosine similarities and their sum are each rounded to bf16 (they are
 // bf16 tensors in the reference); sums inside a reduction are fp32 in a fixed
 // order, so results are deterministic.
 //
-// The sums of the cached sink frames only change when a sink frame is written.
+// The means of the cached sink frames only change when a sink frame is written.
 // A caller that keeps them between calls (frame_sums) has the reduction read
-// the new chunk alone: the decision kernel files the new chunk's sums under the
-// sink frame the append that follows will overwrite, and only frames the
+// the new chunk alone: the deciding workgroup files the new chunk's means under
+// the sink frame the append that follows will overwrite, and only frames the
 // caller marks stale are summed from the cache again.
 //
 // When the q / k RMSNorm is folded into the append the keys arrive raw: a
@@ -46,7 +46,9 @@ constexpr int kLanesPerRow = 16;            // 16 lanes x 8 elements = 128
 constexpr int kTokenLanes = 16;             // 256 threads
 constexpr int kTokenSplits = 8;             // workgroups per (frame, head): token ranges summed apart
 constexpr int kMaxHeads = 64;
-constexpr int kDecideThreads = 1024;
+constexpr int kThreads = kLanesPerRow * kTokenLanes;
+constexpr int kTicketBytes = 256;           // one ticket word per row at the head of the workspace
+static_assert(SDV2_MAX_ROWS * sizeof(int32_t) <= kTicketBytes, "ticket words");
 
 struct SinkSimKernelArgs {
   const void* k_in;
@@ -55,8 +57,9 @@ struct SinkSimKernelArgs {
   const void* v_cache;
   sdv2_stride3 k_in_st, v_in_st, k_st, v_st;
   const double2* freqs;
-  float* sums;                              // [rows][2*sink+2][heads*128][kTokenSplits]: token sums of this call
-  float* kept;                              // [rows][2*sink][heads*128][kTokenSplits] kept between calls, or null
+  int32_t* tickets;                         // [rows], zero between calls
+  float* sums;                              // [rows][2*sink+2][heads][kTokenSplits][128]: token sums of this call
+  float* kept;                              // [rows][2*sink][heads*128] frame means kept between calls, or null
   const void* k_norm_w;                     // RMSNorm weight of k over heads * 128, or null
   float* inv_rms;                           // [rows][tokens]: 1 / rms of every new key token (with k_norm_w)
   float norm_eps;
@@ -72,12 +75,31 @@ struct SinkSimKernelArgs {
   int64_t start_frame[SDV2_MAX_ROWS];
 };
 
-// where the token sums of matrix m (sink K frames, sink V frames, new K, new V) of a row live
+// Token sums travel from the workgroups that form them to the one that
+// decides, which may sit behind another XCD's L2: both sides use relaxed
+// device-scope accesses (the store writes through, the load does not hit in a
+// stale line), ordered by the ticket the deciding workgroup draws last.
+__device__ __forceinline__ void store_coherent(float* p, float x) {
+  __hip_atomic_store(reinterpret_cast<uint32_t*>(p), __float_as_uint(x), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_coherent(const float* p) {
+  return __uint_as_float(
+      __hip_atomic_load(reinterpret_cast<const uint32_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+
+// matrices of a row: sink K frames, sink V frames, new K, new V
 __device__ __forceinline__ float* sums_of(const SinkSimKernelArgs& a, int row, int m) {
-  const int64_t width = static_cast<int64_t>(a.heads) * 128 * kTokenSplits;
+  return a.sums + (static_cast<int64_t>(row) * (2 * a.sink_frames + 2) + m) * a.heads * (kTokenSplits * 128);
+}
+__device__ __forceinline__ float* kept_of(const SinkSimKernelArgs& a, int row, int m) {
+  return a.kept + (static_cast<int64_t>(row) * 2 * a.sink_frames + m) * a.heads * 128;
+}
+// is matrix m summed over its tokens in this call?  (The new chunk always; a
+// sink frame unless its mean is kept and the caller vouches for it.)
+__device__ __forceinline__ bool summed_now(const SinkSimKernelArgs& a, int row, int m) {
   const int sink = a.sink_frames;
-  if (a.kept && m < 2 * sink) return a.kept + (static_cast<int64_t>(row) * 2 * sink + m) * width;
-  return a.sums + (static_cast<int64_t>(row) * (2 * sink + 2) + m) * width;
+  if (m >= 2 * sink || !a.kept) return true;
+  return (a.stale[row] >> (m < sink ? m : m - sink)) & 1u;
 }
 
 template <typename T>
@@ -89,14 +111,183 @@ __device__ __forceinline__ float round_to_storage<uint16_t>(float x) {
 template <>
 __device__ __forceinline__ float round_to_storage<float>(float x) { return x; }
 
+// Frame means from the token sums, cosine similarities, their average, the
+// decision: run by the one workgroup of a row that finished its sums last.  A
+// thread owns kCols columns (columns past the width are clamped and weighted
+// with zero instead of branched around, so all loads of a frame are issued
+// together).  Every dot product is reduced inside its wave as soon as it is
+// formed and the per-wave results wait in LDS, so nothing but loads and
+// arithmetic sits between two frames; the workgroup synchronises once, before
+// the tail.
+template <typename T, int kCols>
+__device__ __forceinline__ void decide(const SinkSimKernelArgs& a, int row) {
+  constexpr int kWaves = kThreads / 64;
+  __shared__ float wave_part[SDV2_MAX_SINK_FRAMES + 1][kWaves][4];
+  __shared__ float sims[SDV2_MAX_SINK_FRAMES];
+  const int sink = a.sink_frames;
+  const int width = a.heads * 128;
+  const float inv_tokens = 1.0f / static_cast<float>(a.tokens);
+  constexpr float kEps = 1e-8f;             // torch.cosine_similarity default
+  // column i of this thread, and its weight (0 past the width)
+  auto col = [&](int i) {
+    const int c = static_cast<int>(threadIdx.x) + i * kThreads;
+    return c < width ? c : width - 1;
+  };
+  auto live = [&](int i) { return static_cast<int>(threadIdx.x) + i * kThreads < width ? 1.f : 0.f; };
+  // means of matrix m at this thread's columns: the token ranges in order and
+  // the rounding of a stored mean, or the mean kept from an earlier call.  The
+  // token sums are fetched for eight columns at a time (64 loads in flight).
+  auto means = [&](int m, float (&out)[kCols]) {
+    if (summed_now(a, row, m)) {
+      const float* p = sums_of(a, row, m);
+      constexpr int kChunk = 8;
+#pragma unroll
+      for (int i0 = 0; i0 < kCols; i0 += kChunk) {
+        float part[kChunk][kTokenSplits];
+#pragma unroll
+        for (int i = 0; i < kChunk; ++i)
+#pragma unroll
+          for (int j = 0; j < kTokenSplits; ++j)
+            if (i0 + i < kCols)
+              part[i][j] = load_coherent(p + ((col(i0 + i) >> 7) * kTokenSplits + j) * 128 + (col(i0 + i) & 127));
+#pragma unroll
+        for (int i = 0; i < kChunk; ++i) {
+          if (i0 + i >= kCols) continue;
+          float sum = 0.f;
+#pragma unroll
+          for (int j = 0; j < kTokenSplits; ++j) sum += part[i][j];
+          out[i0 + i] = round_to_storage<T>(sum * inv_tokens);
+        }
+      }
+      if (a.kept && m < 2 * sink) {
+        float* keep = kept_of(a, row, m);
+#pragma unroll
+        for (int i = 0; i < kCols; ++i) keep[col(i)] = out[i];      // (clamped columns repeat the last one's value)
+      }
+    } else {
+      const float* keep = kept_of(a, row, m);
+#pragma unroll
+      for (int i = 0; i < kCols; ++i) out[i] = keep[col(i)];
+    }
+  };
+  // this wave's share of four sums, in a fixed order, parked in LDS
+  auto park = [&](int slot, float (&x)[4]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) x[i] += __shfl_xor(x[i], off, 64);
+    if ((threadIdx.x & 63) == 0)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) wave_part[slot][threadIdx.x >> 6][i] = x[i];
+  };
+  auto total = [&](int slot, int i) {
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) sum += wave_part[slot][w][i];
+    return sum;
+  };
+
+  // Sink frames are taken kBatch at a time, and the first batch is requested
+  // ahead of the new chunk's sums: loads return in order, so nothing the dot
+  // products need is still on its way when the sums have arrived.  (A batch that
+  // reaches past the last frame repeats it; its results are dropped.)
+  constexpr int kBatch = kCols <= 8 ? 4 : (kCols <= 20 ? 2 : 1);
+  float ks[kBatch][kCols], vs[kBatch][kCols];
+  auto fetch_frames = [&](int j0) {
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int j = j0 + b < sink ? j0 + b : sink - 1;
+      means(j, ks[b]);
+      means(sink + j, vs[b]);
+    }
+  };
+  fetch_frames(0);
+  float k_new[kCols], v_new[kCols];
+  means(2 * sink, k_new);
+  means(2 * sink + 1, v_new);
+  float n[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < kCols; ++i) {
+    n[0] += k_new[i] * k_new[i] * live(i);
+    n[1] += v_new[i] * v_new[i] * live(i);
+  }
+  park(sink, n);
+  for (int j0 = 0; j0 < sink; j0 += kBatch) {
+    if (j0 > 0) fetch_frames(j0);
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      float d[4] = {0.f, 0.f, 0.f, 0.f};    // k.k_new, |k|^2, v.v_new, |v|^2
+#pragma unroll
+      for (int i = 0; i < kCols; ++i) {
+        d[0] += ks[b][i] * k_new[i] * live(i);
+        d[1] += ks[b][i] * ks[b][i] * live(i);
+        d[2] += vs[b][i] * v_new[i] * live(i);
+        d[3] += vs[b][i] * vs[b][i] * live(i);
+      }
+      if (j0 + b < sink) park(j0 + b, d);
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < sink) {
+    const int j = threadIdx.x;
+    const float k_new_norm = fmaxf(sqrtf(total(sink, 0)), kEps);
+    const float v_new_norm = fmaxf(sqrtf(total(sink, 1)), kEps);
+    const float cos_k = round_to_storage<T>(total(j, 0) / (fmaxf(sqrtf(total(j, 1)), kEps) * k_new_norm));
+    const float cos_v = round_to_storage<T>(total(j, 2) / (fmaxf(sqrtf(total(j, 3)), kEps) * v_new_norm));
+    const float sim = round_to_storage<T>(cos_k + cos_v) * 0.5f;
+    a.similarity[row * sink + j] = sim;
+    sims[j] = sim;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float best = sims[0];
+    int best_frame = 0;
+    for (int j = 1; j < sink; ++j)
+      if (sims[j] < best) {                   // first minimum, as torch.argmin
+        best = sims[j];
+        best_frame = j;
+      }
+    const int frame = best < round_to_storage<T>(a.threshold) ? best_frame : -1;
+    a.refresh[row] = frame;
+    sims[0] = __int_as_float(frame);          // (for the hand-over of the kept means below)
+    // The refreshed sink frame goes to the head of the row's eviction queue
+    // (causal_model.py:297-299); a call on the evict branch then writes its
+    // one-frame chunk at [(frame + 1) * tokens - tokens, (frame + 1) * tokens).
+    if (a.dst_override)
+      a.dst_override[row] = frame >= 0 && ((a.override_rows >> row) & 1u) ? static_cast<int64_t>(frame) * a.tokens : -1;
+  }
+  if (a.kept) {
+    // The append that follows overwrites a sink frame when the row evicts into
+    // the frame just chosen, or when the host's plan (a filling call) lands
+    // there: the new chunk's means become that frame's kept means.
+    __syncthreads();
+    const int chosen = __float_as_int(sims[0]);
+    const bool evicting = (a.override_rows >> row) & 1u;
+    const int target = evicting && a.dst_override && chosen >= 0 ? chosen : a.planned_frame[row];
+    if (target >= 0 && target < sink) {
+      float* keep_k = kept_of(a, row, target);
+      float* keep_v = kept_of(a, row, sink + target);
+#pragma unroll
+      for (int i = 0; i < kCols; ++i) {
+        keep_k[col(i)] = k_new[i];
+        keep_v[col(i)] = v_new[i];
+      }
+    }
+  }
+}
+
 // grid (heads, 2*sink+2, rows * kTokenSplits): one workgroup sums one head's
 // 128 columns of one frame over one eighth of its tokens.  (One workgroup per
 // frame and head would leave most of the chip idle: 96 workgroups for three
-// sink frames of twelve heads.)
-template <typename T>
-__global__ __launch_bounds__(kLanesPerRow * kTokenLanes)
-void sink_frame_sum_kernel(const SinkSimKernelArgs a) {
+// sink frames of twelve heads.)  Then it draws its row's ticket, after its
+// sums have been acknowledged by memory; the workgroup that draws the last one
+// finds every sum of the row in memory, decides, and leaves the ticket at zero
+// for the next call.
+template <typename T, int kCols>
+__global__ __launch_bounds__(kThreads)
+void sink_similarity_kernel(const SinkSimKernelArgs a) {
   __shared__ float part[kTokenLanes][kLanesPerRow * 8];
+  __shared__ int is_last;
   const int lane = threadIdx.x & (kLanesPerRow - 1);
   const int tl = threadIdx.x >> 4;
   const int head = blockIdx.x;
@@ -108,8 +299,8 @@ void sink_frame_sum_kernel(const SinkSimKernelArgs a) {
   const bool is_new = m >= 2 * sink;
   const bool is_k = is_new ? (m == 2 * sink) : (m < sink);
   const int frame = is_new ? 0 : (m < sink ? m : m - sink);
-  // a kept frame sum stands until the caller calls it stale
-  if (!is_new && a.kept && !((a.stale[row] >> frame) & 1u)) return;
+  // a kept frame mean stands until the caller calls it stale
+  if (!summed_now(a, row, m)) return;
   const sdv2_stride3 st = is_new ? (is_k ? a.k_in_st : a.v_in_st) : (is_k ? a.k_st : a.v_st);
   const T* base = static_cast<const T*>(is_new ? (is_k ? a.k_in : a.v_in) : (is_k ? a.k_cache : a.v_cache));
   base += row * st.row + static_cast<int64_t>(frame) * a.tokens * st.token + head * st.head + lane * 8;
@@ -178,12 +369,26 @@ void sink_frame_sum_kernel(const SinkSimKernelArgs a) {
   for (int i = 0; i < 8; ++i) part[tl][lane * 8 + i] = acc[i];
   __syncthreads();
   if (threadIdx.x < kLanesPerRow * 8) {
-    float s = 0.f;
+    float sum = 0.f;
 #pragma unroll
-    for (int j = 0; j < kTokenLanes; ++j) s += part[j][threadIdx.x];
-    // the token ranges of one column sit side by side, so the decision kernel fetches them with two 16-byte loads
-    sums_of(a, row, m)[static_cast<int64_t>(head * 128 + threadIdx.x) * kTokenSplits + split] = s;
+    for (int j = 0; j < kTokenLanes; ++j) sum += part[j][threadIdx.x];
+    store_coherent(sums_of(a, row, m) + (head * kTokenSplits + split) * 128 + threadIdx.x, sum);
   }
+  __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0): the stores have been acknowledged
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    // workgroups of this row that sum anything in this call
+    int matrices = 2;
+    for (int f = 0; f < sink; ++f) matrices += summed_now(a, row, f) ? 2 : 0;
+    const int expected = matrices * a.heads * kTokenSplits;
+    const int drawn = __hip_atomic_fetch_add(a.tickets + row, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int last = drawn == expected - 1;
+    if (last) __hip_atomic_store(a.tickets + row, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    is_last = last;
+  }
+  __syncthreads();
+  if (!is_last) return;
+  decide<T, kCols>(a, row);
 }
 
 // grid (tokens / 4, 1, rows): one wave per new key token takes 1 / sqrt(mean(k^2) + eps)
@@ -211,138 +416,6 @@ void key_inv_rms_kernel(const SinkSimKernelArgs a) {
         1.0f / sqrtf(ssq_k / static_cast<float>(a.heads * 128) + a.norm_eps);
 }
 
-// grid (rows): frame means from the partial sums, cosine similarities, their
-// average, the decision.  One workgroup of 1024 threads per row; a thread owns
-// kCols columns (columns past the width are clamped and weighted with zero
-// instead of branched around, so all loads of a frame are issued together).
-// Every dot product is reduced inside its wave as soon as it is formed and the
-// per-wave results wait in LDS, so nothing but loads and arithmetic sits
-// between two frames; the workgroup synchronises once, before the tail.
-template <typename T, int kCols>
-__global__ __launch_bounds__(kDecideThreads)
-void sink_decide_kernel(const SinkSimKernelArgs a) {
-  constexpr int kWaves = kDecideThreads / 64;
-  __shared__ float wave_part[SDV2_MAX_SINK_FRAMES + 1][kWaves][4];
-  __shared__ float sims[SDV2_MAX_SINK_FRAMES];
-  const int row = blockIdx.x;
-  const int sink = a.sink_frames;
-  const int width = a.heads * 128;
-  const float inv_tokens = 1.0f / static_cast<float>(a.tokens);
-  constexpr float kEps = 1e-8f;             // torch.cosine_similarity default
-  int col[kCols];
-  float live[kCols];
-#pragma unroll
-  for (int i = 0; i < kCols; ++i) {
-    const int c = threadIdx.x + i * kDecideThreads;
-    col[i] = c < width ? c : width - 1;
-    live[i] = c < width ? 1.f : 0.f;
-  }
-  // means of frame m at this thread's columns: the token ranges in order, then the rounding of a stored mean
-  auto means = [&](int m, float (&out)[kCols]) {
-    const float* p = sums_of(a, row, m);
-    float4 part[kCols][kTokenSplits / 4];
-#pragma unroll
-    for (int i = 0; i < kCols; ++i)
-#pragma unroll
-      for (int j = 0; j < kTokenSplits / 4; ++j)
-        part[i][j] = *reinterpret_cast<const float4*>(p + static_cast<int64_t>(col[i]) * kTokenSplits + 4 * j);
-#pragma unroll
-    for (int i = 0; i < kCols; ++i) {
-      float s = 0.f;
-#pragma unroll
-      for (int j = 0; j < kTokenSplits / 4; ++j) s = (((s + part[i][j].x) + part[i][j].y) + part[i][j].z) + part[i][j].w;
-      out[i] = round_to_storage<T>(s * inv_tokens) * live[i];
-    }
-  };
-  // this wave's share of four sums, in a fixed order, parked in LDS
-  auto park = [&](int slot, float (&x)[4]) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int off = 32; off > 0; off >>= 1) x[i] += __shfl_xor(x[i], off, 64);
-    if ((threadIdx.x & 63) == 0)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) wave_part[slot][threadIdx.x >> 6][i] = x[i];
-  };
-  auto total = [&](int slot, int i) {
-    float s = 0.f;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) s += wave_part[slot][w][i];
-    return s;
-  };
-
-  float k_new[kCols], v_new[kCols];
-  means(2 * sink, k_new);
-  means(2 * sink + 1, v_new);
-  float n[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int i = 0; i < kCols; ++i) {
-    n[0] += k_new[i] * k_new[i];
-    n[1] += v_new[i] * v_new[i];
-  }
-  park(sink, n);
-  for (int j = 0; j < sink; ++j) {
-    float ks[kCols], vs[kCols];
-    means(j, ks);
-    means(sink + j, vs);
-    float d[4] = {0.f, 0.f, 0.f, 0.f};      // k.k_new, |k|^2, v.v_new, |v|^2
-#pragma unroll
-    for (int i = 0; i < kCols; ++i) {
-      d[0] += ks[i] * k_new[i];
-      d[1] += ks[i] * ks[i];
-      d[2] += vs[i] * v_new[i];
-      d[3] += vs[i] * vs[i];
-    }
-    park(j, d);
-  }
-  __syncthreads();
-  if (threadIdx.x < sink) {
-    const int j = threadIdx.x;
-    const float k_new_norm = fmaxf(sqrtf(total(sink, 0)), kEps);
-    const float v_new_norm = fmaxf(sqrtf(total(sink, 1)), kEps);
-    const float cos_k = round_to_storage<T>(total(j, 0) / (fmaxf(sqrtf(total(j, 1)), kEps) * k_new_norm));
-    const float cos_v = round_to_storage<T>(total(j, 2) / (fmaxf(sqrtf(total(j, 3)), kEps) * v_new_norm));
-    const float sim = round_to_storage<T>(cos_k + cos_v) * 0.5f;
-    a.similarity[row * sink + j] = sim;
-    sims[j] = sim;
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    float best = sims[0];
-    int best_frame = 0;
-    for (int j = 1; j < sink; ++j)
-      if (sims[j] < best) {                   // first minimum, as torch.argmin
-        best = sims[j];
-        best_frame = j;
-      }
-    const int frame = best < round_to_storage<T>(a.threshold) ? best_frame : -1;
-    a.refresh[row] = frame;
-    sims[0] = __int_as_float(frame);          // (for the hand-over of the kept sums below)
-    // The refreshed sink frame goes to the head of the row's eviction queue
-    // (causal_model.py:297-299); a call on the evict branch then writes its
-    // one-frame chunk at [(frame + 1) * tokens - tokens, (frame + 1) * tokens).
-    if (a.dst_override)
-      a.dst_override[row] = frame >= 0 && ((a.override_rows >> row) & 1u) ? static_cast<int64_t>(frame) * a.tokens : -1;
-  }
-  if (a.kept) {
-    // The append that follows overwrites a sink frame when the row evicts into
-    // the frame just chosen, or when the host's plan (a filling call) lands
-    // there: the new chunk's sums become that frame's kept sums.
-    __syncthreads();
-    const int chosen = __float_as_int(sims[0]);
-    const bool evicting = (a.override_rows >> row) & 1u;
-    const int target = evicting && a.dst_override && chosen >= 0 ? chosen : a.planned_frame[row];
-    if (target >= 0 && target < sink) {
-      const int64_t n4 = static_cast<int64_t>(width) * kTokenSplits / 4;
-      for (int which = 0; which < 2; ++which) {
-        const float4* src = reinterpret_cast<const float4*>(sums_of(a, row, 2 * sink + which));
-        float4* dst = reinterpret_cast<float4*>(sums_of(a, row, which * sink + target));
-        for (int64_t i = threadIdx.x; i < n4; i += kDecideThreads) dst[i] = src[i];
-      }
-    }
-  }
-}
-
 bool stride_ok(const sdv2_stride3& s, int vec) {
   return s.row % vec == 0 && s.token % vec == 0 && s.head % vec == 0;
 }
@@ -359,13 +432,14 @@ size_t sums_bytes(int32_t rows, int32_t heads, int32_t sink_frames) {
 extern "C" size_t sdv2_sink_similarity_workspace_bytes(int32_t rows, int32_t tokens, int32_t heads,
                                                         int32_t sink_frames) {
   if (rows <= 0 || tokens <= 0 || heads <= 0 || sink_frames <= 0) return 0;
-  // token sums of every matrix of the call, then 1 / rms per new key token (used with the norm folded in)
-  return sums_bytes(rows, heads, sink_frames) + static_cast<size_t>(rows) * tokens * sizeof(float);
+  // ticket words, token sums of every matrix of the call, then 1 / rms per new
+  // key token (used with the norm folded in)
+  return kTicketBytes + sums_bytes(rows, heads, sink_frames) + static_cast<size_t>(rows) * tokens * sizeof(float);
 }
 
 extern "C" size_t sdv2_sink_frame_sums_bytes(int32_t rows, int32_t heads, int32_t sink_frames) {
   if (rows <= 0 || heads <= 0 || sink_frames <= 0) return 0;
-  return static_cast<size_t>(rows) * 2 * sink_frames * kTokenSplits * heads * SDV2_HEAD_DIM * sizeof(float);
+  return static_cast<size_t>(rows) * 2 * sink_frames * heads * SDV2_HEAD_DIM * sizeof(float);
 }
 
 extern "C" int sdv2_sink_similarity(const sdv2_sink_sim_params* p) {
@@ -407,8 +481,10 @@ extern "C" int sdv2_sink_similarity(const sdv2_sink_sim_params* p) {
   a.k_in = p->k_in; a.v_in = p->v_in; a.k_cache = p->k_cache; a.v_cache = p->v_cache;
   a.k_in_st = p->k_in_stride; a.v_in_st = p->v_in_stride; a.k_st = p->k_cache_stride; a.v_st = p->v_cache_stride;
   a.freqs = reinterpret_cast<const double2*>(p->freqs);
-  a.sums = static_cast<float*>(p->workspace);
-  a.inv_rms = reinterpret_cast<float*>(static_cast<char*>(p->workspace) + sums_bytes(p->rows, p->heads, p->sink_frames));
+  a.tickets = static_cast<int32_t*>(p->workspace);
+  a.sums = reinterpret_cast<float*>(static_cast<char*>(p->workspace) + kTicketBytes);
+  a.inv_rms = reinterpret_cast<float*>(static_cast<char*>(p->workspace) + kTicketBytes +
+                                       sums_bytes(p->rows, p->heads, p->sink_frames));
   a.kept = p->frame_sums;
   a.k_norm_w = p->k_norm_weight;
   a.norm_eps = p->norm_eps;
@@ -429,12 +505,8 @@ extern "C" int sdv2_sink_similarity(const sdv2_sink_sim_params* p) {
   }
 
   hipStream_t stream = static_cast<hipStream_t>(p->stream);
-  const dim3 block(kLanesPerRow * kTokenLanes);
-  const dim3 grid_mean(p->heads, 2 * p->sink_frames + 2, p->rows * kTokenSplits);
-  const dim3 grid_decide(p->rows);
-  const dim3 decide_block(kDecideThreads);
-  // columns per thread of the decision kernel: 2 up to 16 heads, 8 up to 64
-  const bool wide = p->heads * 128 > 2 * kDecideThreads;
+  const dim3 block(kThreads);
+  const dim3 grid(p->heads, 2 * p->sink_frames + 2, p->rows * kTokenSplits);
   if (p->k_norm_weight) {
     const dim3 grid_rms((p->tokens + 3) / 4, 1, p->rows);
     const int steps = (p->heads + 3) / 4;
@@ -447,14 +519,17 @@ extern "C" int sdv2_sink_similarity(const sdv2_sink_sim_params* p) {
     else if (steps <= 10) launch(std::integral_constant<int, 10>{});
     else launch(std::integral_constant<int, 16>{});
   }
-  if (p->dtype == SDV2_BF16) {
-    sdv2::launch_timed(SDV2_KERNEL_SINK_SUM, sink_frame_sum_kernel<uint16_t>, grid_mean, block, 0, stream, a);
-    if (wide) sdv2::launch_timed(SDV2_KERNEL_SINK_DECIDE, sink_decide_kernel<uint16_t, 8>, grid_decide, decide_block, 0, stream, a);
-    else sdv2::launch_timed(SDV2_KERNEL_SINK_DECIDE, sink_decide_kernel<uint16_t, 2>, grid_decide, decide_block, 0, stream, a);
-  } else {
-    sdv2::launch_timed(SDV2_KERNEL_SINK_SUM, sink_frame_sum_kernel<float>, grid_mean, block, 0, stream, a);
-    if (wide) sdv2::launch_timed(SDV2_KERNEL_SINK_DECIDE, sink_decide_kernel<float, 8>, grid_decide, decide_block, 0, stream, a);
-    else sdv2::launch_timed(SDV2_KERNEL_SINK_DECIDE, sink_decide_kernel<float, 2>, grid_decide, decide_block, 0, stream, a);
-  }
+  // columns per thread of the deciding workgroup: 8 up to 16 heads, 20 up to 40, 32 up to 64
+  auto launch = [&](auto cols_c) {
+    constexpr int kCols = decltype(cols_c)::value;
+    if (p->dtype == SDV2_BF16)
+      sdv2::launch_timed(SDV2_KERNEL_SINK, sink_similarity_kernel<uint16_t, kCols>, grid, block, 0, stream, a);
+    else
+      sdv2::launch_timed(SDV2_KERNEL_SINK, sink_similarity_kernel<float, kCols>, grid, block, 0, stream, a);
+  };
+  const int width = p->heads * SDV2_HEAD_DIM;
+  if (width <= 8 * kThreads) launch(std::integral_constant<int, 8>{});
+  else if (width <= 20 * kThreads) launch(std::integral_constant<int, 20>{});
+  else launch(std::integral_constant<int, 32>{});
   return hipGetLastError() == hipSuccess ? SDV2_OK : SDV2_ERR_LAUNCH;
 }

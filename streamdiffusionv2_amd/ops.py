@@ -416,9 +416,9 @@ def sink_similarity(
     ``k_norm`` = (k norm weight, eps): k is the raw k projection and its
     RMSNorm is applied inside, as :func:`kv_append_rope` with ``qk_norm`` does.
 
-    ``frame_sums`` (from :func:`new_sink_frame_sums`) keeps the token sums of
-    the cached sink frames between calls, so that only the new chunk is read:
-    ``stale_frames[i]`` is a bit mask of the sink frames of row i whose sums
+    ``frame_sums`` (from :func:`new_sink_frame_sums`) keeps the means of the
+    cached sink frames between calls, so that only the new chunk is read:
+    ``stale_frames[i]`` is a bit mask of the sink frames of row i whose means
     must be taken from the cache again (written behind this operator's back,
     or never summed), ``planned_frames[i]`` the sink frame the append that
     follows writes to by the host's plan, or -1.
@@ -440,7 +440,7 @@ def sink_similarity(
     need = lib.sdv2_sink_similarity_workspace_bytes(rows, tokens, heads, sink_frames)
     ws = _SIM_WORKSPACES.get(dev)
     if ws is None or ws.numel() < need:
-        ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
+        ws = torch.zeros(max(need, 1), dtype=torch.uint8, device=dev)      # (its ticket words start at zero)
         _SIM_WORKSPACES[dev] = ws
     similarity = torch.empty((rows, sink_frames), dtype=torch.float32, device=dev)
     if refresh_out is None:
@@ -500,7 +500,7 @@ def sink_similarity(
 
 
 def new_sink_frame_sums(rows: int, heads: int, sink_frames: int, dev) -> torch.Tensor:
-    """The buffer :func:`sink_similarity` keeps the sink frames' token sums in
+    """The buffer :func:`sink_similarity` keeps the sink frames' means in
     between calls (everything in it starts out stale)."""
     n = _capi.lib().sdv2_sink_frame_sums_bytes(rows, heads, sink_frames)
     return torch.empty(max(n // 4, 1), dtype=torch.float32, device=dev)

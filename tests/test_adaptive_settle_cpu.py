@@ -72,7 +72,7 @@ def _patched_path(monkeypatch, script, sink):
         refresh = refresh_out if refresh_out is not None else torch.empty(rows, dtype=torch.int32)
         for i in range(rows):
             refresh[i] = decisions[i]
-            if dst_start_override is not None:      # what sink_decide_kernel stores
+            if dst_start_override is not None:      # what the deciding workgroup of sink_similarity_kernel stores
                 dst_start_override[i] = decisions[i] * k.shape[1] if decisions[i] >= 0 and override_rows[i] else -1
         return None, refresh
 
