@@ -265,13 +265,17 @@ def new_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
     return torch.zeros(max(nbytes, 1), dtype=torch.uint8, device=dev)
 
 
-def _workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
-    """Per-device scratch for split-KV partials, grown on demand and reused
-    (safe for stream-ordered use on one stream: a call is one launch)."""
-    ws = _WORKSPACES.get(dev)
+def _workspace(dev: torch.device, nbytes: int, pool: Optional[dict] = None) -> torch.Tensor:
+    """Scratch for split-KV partials, one buffer per (device, stream), grown on
+    demand and reused.  Calls on one stream run one after another, so they can
+    share a buffer; calls on different streams may overlap in time and must not
+    (their tickets and partial results would mix), so each stream gets its own."""
+    pool = _WORKSPACES if pool is None else pool
+    key = (dev, _stream_ptr(dev))
+    ws = pool.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = new_workspace(dev, nbytes)
-        _WORKSPACES[dev] = ws
+        pool[key] = ws
     return ws
 
 
@@ -438,10 +442,7 @@ def sink_similarity(
         raise RuntimeError(f"cache {tuple(k_cache.shape)} does not match the chunk {tuple(k.shape)}")
     lib = _capi.lib()
     need = lib.sdv2_sink_similarity_workspace_bytes(rows, tokens, heads, sink_frames)
-    ws = _SIM_WORKSPACES.get(dev)
-    if ws is None or ws.numel() < need:
-        ws = torch.zeros(max(need, 1), dtype=torch.uint8, device=dev)      # (its ticket words start at zero)
-        _SIM_WORKSPACES[dev] = ws
+    ws = _workspace(dev, need, _SIM_WORKSPACES)      # (zero-filled: its ticket words start at zero)
     similarity = torch.empty((rows, sink_frames), dtype=torch.float32, device=dev)
     if refresh_out is None:
         refresh = torch.empty((rows,), dtype=torch.int32, device=dev)
@@ -628,6 +629,7 @@ class LayerLauncher:
         at.rows, at.q_tokens, at.heads, at.head_dim = rows, tokens, heads, HEAD_DIM
         self.at, self.at_ref = at, C.byref(at)
         self.span = -1
+        self.workspace_need = 0
         self.out_stride = None
         self.forced_splits = 0                       # 0 = the library's own choice
         self.timers = (None, None)
@@ -675,12 +677,10 @@ class LayerLauncher:
             at.max_seq_len = span
             at.num_splits = self.forced_splits or self.lib.sdv2_swa_attn_default_splits(
                 self.rows, self.tokens, self.heads, span)
-            need = self.lib.sdv2_swa_attn_workspace_bytes(self.rows, self.tokens, self.heads, span, at.num_splits)
-            if need:
-                ws = _workspace(self.dev, need)
-                at.workspace, at.workspace_bytes = ws.data_ptr(), ws.numel()
-        elif at.workspace:
-            ws = _WORKSPACES[self.dev]              # may have been regrown by another shape
+            self.workspace_need = self.lib.sdv2_swa_attn_workspace_bytes(self.rows, self.tokens, self.heads, span,
+                                                                         at.num_splits)
+        if self.workspace_need:
+            ws = _workspace(self.dev, self.workspace_need)      # this stream's; may have been regrown by another shape
             at.workspace, at.workspace_bytes = ws.data_ptr(), ws.numel()
         out = torch.empty((self.rows, self.tokens, self.heads, HEAD_DIM), dtype=torch.bfloat16, device=self.dev)
         if self.out_stride is None:

@@ -265,6 +265,38 @@ def test_one_workspace_serves_changing_shapes(gpu_device):
         assert not ws[:65536].any()                     # the ticket words
 
 
+def test_every_stream_gets_its_own_workspace(gpu_device):
+    """Split calls that overlap in time must not share tickets and partial
+    results: the wrapper keeps one workspace per (device, stream), so calls
+    issued on two streams at once both come out right."""
+    from streamdiffusionv2_amd import ops
+
+    torch.manual_seed(21)
+    rows, S, H, L, sp = 1, 600, 4, 6000, 4
+    data = []
+    for i in range(2):
+        gen = torch.Generator().manual_seed(500 + i)
+        data.append(tuple(torch.randn(rows, n, H, 128, generator=gen).bfloat16() for n in (S, L, L)))
+    on_gpu = [tuple(t.to(gpu_device) for t in d) for d in data]
+    streams = [torch.cuda.Stream(device=gpu_device) for _ in range(2)]
+    torch.cuda.synchronize()
+    got = [[], []]
+    for _ in range(6):                                   # the two streams' launches interleave
+        for i, stream in enumerate(streams):
+            with torch.cuda.stream(stream):
+                q, k, v = on_gpu[i]
+                got[i].append(ops.swa_attention(q, k, v, None, num_splits=sp))
+    torch.cuda.synchronize()
+    keys = [key for key in ops._WORKSPACES if key[0] == gpu_device]
+    assert len({ops._WORKSPACES[(gpu_device, s.cuda_stream)].data_ptr() for s in streams}) == 2, keys
+    for i in range(2):
+        q, k, v = data[i]
+        want = oracle.attention_fp32_reference(q, k, v, [L] * rows)
+        for out in got[i]:
+            assert torch.equal(out, got[i][0])
+            _check(out.cpu(), want)
+
+
 def test_one_extreme_query_row_costs_less_than_a_second_launch(gpu_device):
     """A single query row whose scores leave the fast softmax's range sends one
     wave of one workgroup through the running-maximum pass, not the whole
