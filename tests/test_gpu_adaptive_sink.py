@@ -144,9 +144,10 @@ def test_similarity_operator(gpu_device, dtype, tol, head_major):
 @pytest.mark.gpu
 @pytest.mark.parametrize("heads,sink", [(40, 3), (17, 16), (64, 2), (1, 1)])
 def test_similarity_operator_wide_and_deep(gpu_device, heads, sink):
-    """The decision kernel has a build for up to 16 heads and one for up to 64,
-    and room for 16 sink frames; the slot hand-over is checked on the way
-    (rows 0 and 2 flagged as evicting)."""
+    """The kernel has builds for up to 16, 40 and 64 heads (8, 20 and 32 columns
+    per thread of the deciding workgroup, which takes the sink frames four,
+    two or one at a time) and room for 16 sink frames; the slot hand-over is
+    checked on the way (rows 0 and 2 flagged as evicting)."""
     from streamdiffusionv2_amd import ops, rope
 
     print(f"sink similarity operator: heads={heads} sink={sink}", flush=True)
@@ -259,9 +260,9 @@ def test_stream_with_refresh(gpu_device, seed, rows, look_every_call):
 # --------------------------------------------------------------------------
 # The shipped shape: 480p latent frames of 30 x 52 = 1560 tokens, sink 3,
 # threshold 0.2 (configs/wan_causal_dmd_v2v.yaml:53-56), 12 heads (Wan 1.3B)
-# and 40 heads (Wan 14B).  At this frame size every workgroup of the frame-sum
-# kernel runs its four-tokens-in-flight main loop (195 tokens per workgroup)
-# and 40 heads take the wide build of the decision kernel.
+# and 40 heads (Wan 14B).  At this frame size every workgroup runs its
+# four-tokens-in-flight main loop (195 tokens per workgroup) and 40 heads take
+# the middle build of the kernel (20 columns per deciding thread).
 # --------------------------------------------------------------------------
 PROD_GRID = (1, 30, 52)
 PROD_FT = 1560
