@@ -128,8 +128,7 @@ class RingKVPath:
         if pending is None:
             return
         self._pending = None
-        pending["event"].synchronize()
-        refresh = pending["host"].tolist()
+        refresh = self._await_decision(pending["host"], pending["stream"])
         self._last_refresh = refresh
         plan, tokens, frame_tokens = pending["plan"], pending["tokens"], pending["frame_tokens"]
         sink_tokens = pending["sink_size"] * frame_tokens
@@ -152,21 +151,32 @@ class RingKVPath:
     # kv_idx < ends[q_idx], causal_model.py:670-686).
     block_frames: Optional[int] = None
 
+    # what the pinned decision words hold from the launch until the kernel has written them
+    _NOT_YET = -(2 ** 31)
+
     def _decision_buffers(self, rows: int, dev):
-        """Per path: the device slot override the decision kernel writes, the
-        pinned host copy of the decision and the event that says it arrived."""
+        """Per path: the device slot override the decision kernel writes and
+        the pinned host words it writes the decision to."""
         buf = getattr(self, "_decision", None)
         if buf is None or buf[0].numel() != rows or buf[0].device != dev:
             buf = (torch.full((rows,), -1, dtype=torch.int64, device=dev),
-                   torch.empty((rows,), dtype=torch.int32, pin_memory=True),
-                   torch.cuda.Event())
+                   torch.empty((rows,), dtype=torch.int32, pin_memory=True))
             self._decision = buf
         return buf
 
-    @staticmethod
-    def _mark_decision(event, dev) -> None:
-        """The decision is on the host once the stream has passed this point."""
-        event.record(torch.cuda.current_stream(dev))
+    def _await_decision(self, host: torch.Tensor, stream) -> List[int]:
+        """The decision of the last check, once it is on the host.  Nothing is
+        recorded on the stream for it (an event between the decision kernel and
+        the append costs the stream 6 us per layer): the words are preset to a
+        value no decision takes, the kernel stores straight into them, and only
+        a reader that comes before they have arrived waits for the stream."""
+        refresh = host.tolist()
+        if self._NOT_YET in refresh:
+            stream.synchronize()
+            refresh = host.tolist()
+            if self._NOT_YET in refresh:
+                raise RuntimeError("the adaptive sink decision never arrived: the launch that was to write it failed")
+        return refresh
 
     # Token sums of the cached sink frames, kept between the adaptive checks of
     # this path so that a check reads the new chunk only.  `stale` holds, per
@@ -274,7 +284,8 @@ class RingKVPath:
                 # adaptive sink refresh (causal_model.py:284-299): one fused
                 # reduction on the device, whose decision goes straight to the
                 # append below and, written into pinned memory by the kernel, to the host
-                override, host, event = self._decision_buffers(rows, q.device)
+                override, host = self._decision_buffers(rows, q.device)
+                host.fill_(self._NOT_YET)
                 kept = self._kept_sink_sums(kv_cache, rows, q.shape[2])
                 extra = {}
                 if kept is not None:
@@ -287,8 +298,7 @@ class RingKVPath:
                     k, v, kv_cache["k"], kv_cache["v"], table, (h, w), [c // frame_tokens for c in starts],
                     self.sink_size, self.adapt_sink_thr, dst_start_override=override, override_rows=plan.evicting,
                     refresh_out=host, k_norm=k_norm, **extra)
-                self._mark_decision(event, q.device)
-                self._pending = dict(event=event, host=host, plan=plan, queues=queues_before, starts=list(starts),
+                self._pending = dict(stream=torch.cuda.current_stream(q.device), host=host, plan=plan, queues=queues_before, starts=list(starts),
                                      tokens=q.shape[1], frame_tokens=frame_tokens, sink_size=self.sink_size,
                                      cap=kv_cache["k"].shape[1])
             if not adaptive:
@@ -343,6 +353,10 @@ class RingKVPath:
             return out
 
         except Exception:
+            if self._pending is not None:
+                # a decision kernel may be on its way: let it store its (now unwanted) words
+                # before a later call presets them again
+                self._pending["stream"].synchronize()
             self._evict_idx, self._pending, self._sink_sums = undo[0], None, None
             if undo[1] is not None:
                 kv_cache["current_step"] = undo[1]

@@ -25,10 +25,7 @@ FT = 6            # tokens per frame
 GRID = (1, 2, 3)
 
 
-class _Event:
-    def record(self, stream=None):
-        pass
-
+class _Stream:
     def synchronize(self):
         pass
 
@@ -79,11 +76,11 @@ def _patched_path(monkeypatch, script, sink):
     monkeypatch.setattr(attention.ops, "device_freqs", lambda freqs, dev: None)
     monkeypatch.setattr(attention.ops, "sink_similarity", fake_similarity)
     monkeypatch.setattr(path, "_layer_launcher", lambda *a, **kw: launcher)
-    monkeypatch.setattr(path, "_mark_decision", lambda event, dev: None)
+    monkeypatch.setattr(attention.torch.cuda, "current_stream", lambda dev=None: _Stream())
     monkeypatch.setattr(path, "_kept_sink_sums", lambda kv_cache, rows, heads: None)
     monkeypatch.setattr(path, "_decision_buffers",
                         lambda rows, dev: (torch.full((rows,), -1, dtype=torch.int64),
-                                           torch.empty(rows, dtype=torch.int32), _Event()))
+                                           torch.empty(rows, dtype=torch.int32)))
     return path, launcher
 
 
