@@ -203,8 +203,34 @@ __device__ __forceinline__ void decide(const SinkSimKernelArgs& a, int row) {
   };
   fetch_frames(0);
   float k_new[kCols], v_new[kCols];
-  means(2 * sink, k_new);
-  means(2 * sink + 1, v_new);
+  if constexpr (kCols <= 8) {
+    // few enough columns per thread that the token sums of both new matrices
+    // fit the registers at once: one trip to memory instead of two
+    float part[2][kCols][kTokenSplits];
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+      const float* p = sums_of(a, row, 2 * sink + m);
+#pragma unroll
+      for (int i = 0; i < kCols; ++i)
+#pragma unroll
+        for (int j = 0; j < kTokenSplits; ++j)
+          part[m][i][j] = load_coherent(p + ((col(i) >> 7) * kTokenSplits + j) * 128 + (col(i) & 127));
+    }
+#pragma unroll
+    for (int i = 0; i < kCols; ++i) {
+      float sum_k = 0.f, sum_v = 0.f;
+#pragma unroll
+      for (int j = 0; j < kTokenSplits; ++j) {
+        sum_k += part[0][i][j];
+        sum_v += part[1][i][j];
+      }
+      k_new[i] = round_to_storage<T>(sum_k * inv_tokens);
+      v_new[i] = round_to_storage<T>(sum_v * inv_tokens);
+    }
+  } else {
+    means(2 * sink, k_new);
+    means(2 * sink + 1, v_new);
+  }
   float n[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int i = 0; i < kCols; ++i) {
