@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SDV2KV_ABI_VERSION 9
+#define SDV2KV_ABI_VERSION 10
 #define SDV2_HEAD_DIM 128      /* causal_stream_inference.py:99-100 fixes 128 */
 #define SDV2_MAX_ROWS 16       /* rows (B) per sdv2_kv_append_rope call       */
 #define SDV2_MAX_SINK_FRAMES 16 /* sink frames per sdv2_sink_similarity call  */
@@ -50,8 +50,8 @@ typedef enum sdv2_status {
 
 typedef enum sdv2_dtype {
   SDV2_BF16 = 0,
-  SDV2_F32 = 1                 /* append only (CPU-plumbing config of the     */
-                               /* reference runs fp32); attention is bf16     */
+  SDV2_F32 = 1                 /* the reference's CPU-runnable configuration: */
+                               /* same operators, fp32 storage and arithmetic */
 } sdv2_dtype;
 
 /* element strides of a [rows, tokens, heads, 128] tensor */
@@ -162,10 +162,10 @@ int sdv2_kv_append_rope(const sdv2_append_params* p);
  * (causal_model.py:253-266 rotates q only to feed it to this operator).
  * ---------------------------------------------------------------------- */
 typedef struct sdv2_attn_params {
-  const void* q;               /* [B,S,H,128] bf16 (roped)                     */
-  const void* k_cache;         /* [B,L,H,128] bf16 view of the cache           */
+  const void* q;               /* [B,S,H,128] bf16 or fp32, see dtype (roped)  */
+  const void* k_cache;         /* [B,L,H,128] view of the cache, same dtype    */
   const void* v_cache;
-  void* out;                   /* [B,S,H,128] bf16                             */
+  void* out;                   /* [B,S,H,128], same dtype                      */
   const int32_t* seq_lens;     /* device int32 [B]; NULL = every row uses L    */
   sdv2_stride3 q_stride, k_stride, v_stride, out_stride;
   int32_t rows, q_tokens, heads, head_dim;        /* B, S, H, 128              */
@@ -195,6 +195,12 @@ typedef struct sdv2_attn_params {
   int32_t rope_freq_rows;
   int32_t rope_grid_h, rope_grid_w;
   const int64_t* rope_start_frame; /* host [B]                                     */
+  /* sdv2_dtype of q, both caches and out.  SDV2_BF16 (0): the matrix-core
+   * kernel.  SDV2_F32: what the reference's fallback operator computes on fp32
+   * tensors (causal_model.py:111-157) - products, sums and softmax in fp32,
+   * one key range (num_splits, workspace and rope_freqs must be unset: fp32
+   * queries arrive rotated), strides in multiples of 4 elements.             */
+  int32_t dtype;
 } sdv2_attn_params;
 
 /* number of key-range splits the library would pick for this shape */

@@ -12,7 +12,7 @@ from typing import Optional
 
 LIB_PATH = Path(__file__).resolve().parent / "_lib" / "libsdv2kv.so"
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 HEAD_DIM = 128
 MAX_ROWS = 16
 
@@ -99,6 +99,7 @@ class AttnParams(C.Structure):
         ("rope_freq_rows", C.c_int32),
         ("rope_grid_h", C.c_int32), ("rope_grid_w", C.c_int32),
         ("rope_start_frame", C.POINTER(C.c_int64)),
+        ("dtype", C.c_int32),
     ]
 
 

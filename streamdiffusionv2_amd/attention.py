@@ -339,15 +339,9 @@ class RingKVPath:
                 dst_start_override=override,
             )
             mask = dict(chunk_key_start=list(plan.dst_start), mask_block_tokens=mask_tokens) if mask_tokens else {}
-            if roped_q.dtype == torch.bfloat16:
-                out = ops.swa_attention(roped_q, kv_cache["k"][:, :span], kv_cache["v"][:, :span], seq, **mask)
-            else:
-                # fp32 storage is a plumbing mode (the reference's CPU-runnable
-                # configuration): RoPE, cache and indices stay fp32 and bit-exact,
-                # the attention kernel computes in bf16 on down-cast copies.
-                out = ops.swa_attention(
-                    roped_q.bfloat16(), kv_cache["k"][:, :span].bfloat16(), kv_cache["v"][:, :span].bfloat16(), seq, **mask
-                ).to(roped_q.dtype)
+            # (fp32 storage, the reference's CPU-runnable configuration, is computed in
+            # fp32 throughout by a plain kernel; the matrix-core kernel is the bf16 one)
+            out = ops.swa_attention(roped_q, kv_cache["k"][:, :span], kv_cache["v"][:, :span], seq, **mask)
             if return_roped_query:
                 return out, roped_q
             return out

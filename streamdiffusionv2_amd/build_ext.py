@@ -16,7 +16,7 @@ REPO_ROOT = PKG_DIR.parent
 CSRC = PKG_DIR / "csrc"
 LIB_DIR = PKG_DIR / "_lib"
 LIB_PATH = LIB_DIR / "libsdv2kv.so"
-SOURCES = ["sdv2kv_api.hip", "kv_append_rope.hip", "swa_attn_fwd.hip", "sink_similarity.hip",
+SOURCES = ["sdv2kv_api.hip", "kv_append_rope.hip", "swa_attn_fwd.hip", "swa_attn_fwd_f32.hip", "sink_similarity.hip",
            "cache_relayout.hip"]
 
 # -packed-fp32-ops is switched off: the compiler would otherwise form

@@ -6,7 +6,12 @@
 #include <hip/hip_ext.h>
 #include <stdint.h>
 
+struct sdv2_attn_params;
+
 namespace sdv2 {
+
+// sdv2_swa_attn_fwd for fp32 tensors (swa_attn_fwd_f32.hip): fp32 arithmetic throughout, unsplit
+int attn_fwd_f32(const sdv2_attn_params* p);
 
 // Measurement hooks (sdv2kv_profile.h), kept per calling thread in
 // sdv2kv_api.hip: the event pair armed for the next launch of a kernel (taken

@@ -1166,6 +1166,8 @@ extern "C" int sdv2_swa_attn_fwd_static(const sdv2_attn_params* p) {
 namespace {
 
 int attn_fwd(const sdv2_attn_params* p, void* workspace, size_t workspace_bytes) {
+  if (p->dtype == SDV2_F32) return sdv2::attn_fwd_f32(p);        // fp32 arithmetic, one key range: no workspace
+  if (p->dtype != SDV2_BF16) return SDV2_ERR_UNSUPPORTED;
   if (p->head_dim != kD) return SDV2_ERR_UNSUPPORTED;
   if (p->rows < 0 || p->q_tokens < 0 || p->heads <= 0 || p->max_seq_len < 0) return SDV2_ERR_INVALID_ARG;
   if (p->rows == 0 || p->q_tokens == 0) return SDV2_OK;

@@ -322,28 +322,37 @@ def swa_attention(
     whole call then allocates nothing.
 
     q [B,S,H,128] bf16; k_cache/v_cache [B,L,H,128] bf16 views with any row /
-    token / head strides; seq_lens int32 [B] on the device (None = L).
+    token / head strides; seq_lens int32 [B] on the device (None = L).  All
+    three may be fp32 instead (the reference's CPU-runnable configuration): the
+    result is then computed in fp32 throughout, by a plain kernel that walks the
+    whole key range (q rotated beforehand, ``num_splits`` ignored).
     With ``mask_block_tokens`` = b in (0, S) and ``chunk_key_start`` (int32 [B]
     on the device, or host ints: where each row's own chunk sits in the cache)
     query token t does not see the chunk's later blocks
     [start + (t // b + 1) * b, start + S).
     """
     dev = _require_gpu(q, k_cache, v_cache, seq_lens, out, workspace)
-    if q.dtype != torch.bfloat16 or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16:
-        raise RuntimeError("swa_attention computes in bf16; got %s/%s/%s" % (q.dtype, k_cache.dtype, v_cache.dtype))
+    if q.dtype not in _DTYPES or k_cache.dtype != q.dtype or v_cache.dtype != q.dtype:
+        raise RuntimeError("swa_attention takes q and both caches in one dtype, bf16 or fp32; got %s/%s/%s"
+                           % (q.dtype, k_cache.dtype, v_cache.dtype))
+    fp32 = q.dtype == torch.float32
+    if fp32 and (rope is not None or static_scratch):
+        raise RuntimeError("fp32 attention takes rotated queries and one key range (no rope=, no static_scratch=)")
     rows, q_tokens, heads, _ = q.shape
     if k_cache.shape[0] != rows or k_cache.shape[2] != heads or v_cache.shape != k_cache.shape:
         raise RuntimeError(f"cache view {tuple(k_cache.shape)} / {tuple(v_cache.shape)} does not match q {tuple(q.shape)}")
     if seq_lens is not None and (seq_lens.dtype != torch.int32 or seq_lens.numel() != rows or not seq_lens.is_contiguous()):
         raise RuntimeError("seq_lens must be a contiguous int32 tensor with one entry per row")
     if out is None:
-        out = torch.empty((rows, q_tokens, heads, HEAD_DIM), dtype=torch.bfloat16, device=dev)
-    elif out.dtype != torch.bfloat16 or tuple(out.shape) != tuple(q.shape):
-        raise RuntimeError("out must be bf16 with q's shape")
+        out = torch.empty((rows, q_tokens, heads, HEAD_DIM), dtype=q.dtype, device=dev)
+    elif out.dtype != q.dtype or tuple(out.shape) != tuple(q.shape):
+        raise RuntimeError("out must have q's dtype and shape")
 
     lib = _capi.lib()
     max_seq_len = k_cache.shape[1]
-    if num_splits <= 0:
+    if fp32:
+        num_splits = 1          # the fp32 kernel walks the whole key range
+    elif num_splits <= 0:
         num_splits = lib.sdv2_swa_attn_default_splits(rows, q_tokens, heads, max_seq_len)
     need = 0 if static_scratch else lib.sdv2_swa_attn_workspace_bytes(rows, q_tokens, heads, max_seq_len, num_splits)
     if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
@@ -358,6 +367,7 @@ def swa_attention(
     p.rows, p.q_tokens, p.heads, p.head_dim = rows, q_tokens, heads, HEAD_DIM
     p.max_seq_len = max_seq_len
     p.num_splits = num_splits
+    p.dtype = _DTYPES[q.dtype]
     p.softmax_scale = float(softmax_scale) if softmax_scale else 0.0
     if need:
         p.workspace = workspace.data_ptr()

@@ -190,7 +190,7 @@ def test_plain_c_caller(tmp_path):
     import re
 
     for c_name, binding, last in (("sdv2_append_params", _capi.AppendParams, "dst_start_override"),
-                                  ("sdv2_attn_params", _capi.AttnParams, "rope_start_frame"),
+                                  ("sdv2_attn_params", _capi.AttnParams, "dtype"),
                                   ("sdv2_sink_sim_params", _capi.SinkSimParams, "planned_frame"),
                                   ("sdv2_relayout_params", _capi.RelayoutParams, "global_end_shift")):
         m = re.search(rf"layout {c_name} size=(\d+) stream=(\d+) {last}=(\d+)", run.stdout)

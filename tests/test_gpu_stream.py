@@ -26,7 +26,7 @@ def _bits(t):
 
 
 def _run(w, gpu_device, layers, calls, sample_rows=None, full_compare_at=None, pool=None, first_layer=0,
-         attention_every=1):
+         attention_every=1, max_abs=MAX_ABS, mean_abs=MEAN_ABS):
     """`pool` (workloads.InputPool) replaces the per-call random draw for long
     streams; `first_layer` offsets the layer number that selects the inputs;
     with `attention_every` = n the attention output is checked on every n-th
@@ -89,8 +89,8 @@ def _run(w, gpu_device, layers, calls, sample_rows=None, full_compare_at=None, p
             assert torch.isfinite(err).all()
             worst_max = max(worst_max, err.max().item())
             worst_mean = max(worst_mean, err.mean().item())
-            assert err.max().item() <= MAX_ABS, (call, layer, err.max().item())
-            assert err.mean().item() <= MEAN_ABS, (call, layer, err.mean().item())
+            assert err.max().item() <= max_abs, (call, layer, err.max().item())
+            assert err.mean().item() <= mean_abs, (call, layer, err.mean().item())
     print(f"  worst max-abs {worst_max:.3e}, worst mean-abs {worst_mean:.3e}", flush=True)
 
 
@@ -99,9 +99,9 @@ def _small(w, **kw):
 
 
 def test_c1_fp32_plumbing(gpu_device):
-    # fp32 storage: append and ring state are bit-exact in fp32; the attention
-    # kernel computes in bf16 on a down-cast copy and is held to the same tolerance
-    _run(workloads.WORKLOADS[1], gpu_device, layers=1, calls=10)
+    # fp32 storage: append and ring state are bit-exact in fp32, and the attention is
+    # computed in fp32 throughout, so it is held to fp32 agreement with the fp32 oracle
+    _run(workloads.WORKLOADS[1], gpu_device, layers=1, calls=10, max_abs=5e-6, mean_abs=5e-7)
 
 
 @pytest.mark.parametrize("cfg,grid,layers,calls", [
