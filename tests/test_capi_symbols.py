@@ -99,6 +99,17 @@ def test_argument_validation_without_gpu():
     assert lib.sdv2_swa_attn_fwd(C.byref(a)) == _capi.SDV2_ERR_UNSUPPORTED
     a.head_dim, a.rows, a.q_tokens, a.heads, a.max_seq_len = 128, 1, 4, 1, 8
     assert lib.sdv2_swa_attn_fwd(C.byref(a)) == _capi.SDV2_ERR_INVALID_ARG     # null tensors
+    a.dtype = 7
+    assert lib.sdv2_swa_attn_fwd(C.byref(a)) == _capi.SDV2_ERR_UNSUPPORTED     # neither bf16 nor fp32
+    a.dtype = _capi.DTYPE_F32
+    assert lib.sdv2_swa_attn_fwd(C.byref(a)) == _capi.SDV2_ERR_INVALID_ARG     # fp32: null tensors all the same
+    a.q, a.k_cache, a.v_cache, a.out = 256, 512, 768, 1024
+    for st in (a.q_stride, a.k_stride, a.v_stride, a.out_stride):
+        st.row, st.token, st.head = 1024, 128, 128
+    a.rope_freqs = 2048
+    assert lib.sdv2_swa_attn_fwd(C.byref(a)) == _capi.SDV2_ERR_UNSUPPORTED     # fp32 queries arrive rotated
+    a.rope_freqs, a.q_stride.token = None, 130
+    assert lib.sdv2_swa_attn_fwd(C.byref(a)) == _capi.SDV2_ERR_INVALID_ARG     # fp32 strides in multiples of 4
     assert b"workspace" in lib.sdv2_status_string(_capi.SDV2_ERR_WORKSPACE)
     with pytest.raises(RuntimeError, match="status -3"):
         _capi.check(_capi.SDV2_ERR_OUT_OF_RANGE, "x")
