@@ -145,7 +145,9 @@ int sdv2_kv_append_rope(const sdv2_append_params* p);
  *   out[i] = softmax(q[i] k_cache[i,:seq_lens[i]]^T / sqrt(128)) v_cache[i,:seq_lens[i]]
  * with no mask inside the chunk (causal=False) unless one is asked for (see
  * mask_block_tokens) and keys at or beyond seq_lens[i] ignored.  bf16 in, fp32
- * accumulation, bf16 out.
+ * accumulation, bf16 out - or, with dtype = SDV2_F32, fp32 tensors and fp32
+ * arithmetic throughout (what the fallback computes on the reference's CPU-
+ * runnable fp32 configuration).
  *
  * Long caches are split over key ranges to fill the 256 CUs; partial results
  * go through `workspace` (size from sdv2_swa_attn_workspace_bytes) and the
