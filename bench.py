@@ -704,8 +704,8 @@ def main():
 
     w = workloads.WORKLOADS[args.workload]
     if w.dtype != torch.bfloat16:
-        print("the GPU attention kernel computes in bf16; workload 1 is the CPU-plumbing parity case, "
-              "not a bench line", file=sys.stderr)
+        print("workload 1 is the reference's CPU-runnable parity case (fp32 tensors, checked by the GPU tests), "
+              "not a bench line; the measured workloads are 2-5", file=sys.stderr)
         sys.exit(2)
     if args.record_traffic:
         record_traffic(args, w)
