@@ -147,6 +147,9 @@ def parse_args():
     ap.add_argument("--softmax-range", action="store_true",
                     help="also time the attention launch with the queries scaled up until rows leave the range the fast "
                          "softmax covers and waves redo their block with the running-maximum recurrence")
+    ap.add_argument("--skip-mfma-ceiling", action="store_true",
+                    help="do not run the library's own MFMA / LDS / softmax instruction streams (what this box sustains "
+                         "on the attention kernel's instruction mix)")
     ap.add_argument("--skip-mfma-reference", action="store_true",
                     help="do not time the vendor bf16 GEMM that shows what this box sustains on MFMA")
     return ap.parse_args()
@@ -313,6 +316,56 @@ def mfma_reference(n=8192, iters=20):
         e1.record()
         torch.cuda.synchronize()
         out[kind] = 2 * n ** 3 / (e0.elapsed_time(e1) / iters) / 1e9
+    return out
+
+
+def mfma_ceiling_section(achieved_tflops):
+    """What this box sustains on the attention kernel's own instruction streams
+    (the library's sdv2_profile_mfma_stream, random operands, one workgroup per
+    CU): the matrix instructions alone; with the LDS fragment reads of the
+    kernel's 32-rows-per-wave blocking; with those of a 64-rows-per-wave
+    blocking; and with the softmax instructions, tile transfers and per-tile
+    barrier of the attention loop.  Context for roofline.frac: the published
+    2.5 PFLOP/s is not what a power-limited chip holds on toggling operands."""
+    import ctypes as C
+
+    from streamdiffusionv2_amd import _capi
+
+    lib = _capi.lib()
+    dev = torch.device("cuda:0")
+    nbytes = lib.sdv2_profile_mfma_stream_bytes()
+    out = {"unit": "TFLOP/s", "operands": "random bf16, N(0, 0.3)", "workgroups": 256}
+    stream = torch.cuda.current_stream(dev).cuda_stream
+    flops = C.c_double()
+    names = (("mfma_only_registers", _capi.STREAM_REGISTERS), ("lds_reads_32_rows_per_wave", _capi.STREAM_LDS_32_ROWS),
+             ("lds_reads_64_rows_per_wave", _capi.STREAM_LDS_64_ROWS), ("attention_loop_mix", _capi.STREAM_ATTENTION_MIX))
+    for kind in ("random", "zeros"):
+        if kind == "random":
+            buf = (torch.randn(nbytes // 2, device=dev) * 0.3).bfloat16()
+        else:
+            buf = torch.zeros(nbytes // 2, device=dev, dtype=torch.bfloat16)
+        for name, mode in names:
+            if kind == "zeros" and mode not in (_capi.STREAM_REGISTERS, _capi.STREAM_ATTENTION_MIX):
+                continue
+
+            def launch():
+                _capi.check(lib.sdv2_profile_mfma_stream(mode, buf.data_ptr(), nbytes, 150, stream, C.byref(flops)),
+                            "sdv2_profile_mfma_stream")
+
+            for _ in range(40):             # long enough for the clock to settle under the load
+                launch()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(80):
+                launch()
+            e1.record()
+            torch.cuda.synchronize()
+            rate = flops.value * 80 / (e0.elapsed_time(e1) * 1e-3) / 1e12
+            out[name if kind == "random" else name + "_zeros"] = rate
+        del buf
+    out["attention_kernel_vs_attention_loop_mix"] = achieved_tflops / out["attention_loop_mix"]
+    out["frac_of_peak_attention_loop_mix"] = out["attention_loop_mix"] / PEAK_BF16_TFLOPS
     return out
 
 
@@ -652,7 +705,12 @@ def cpu_baseline(args, w):
     from oracle import sdv2_oracle as oracle
     from streamdiffusionv2_amd import workloads
 
-    threads = min(os.cpu_count() or 1, 16)
+    # The reference's CPU path runs on torch's intra-op pool.  A one-GPU box of this pool gives a
+    # job a share of 16 host cores whatever os.cpu_count() shows (OMP_NUM_THREADS says so there):
+    # the thread count follows that share, and both numbers are reported.
+    host_cpus = os.cpu_count() or 1
+    share = int(os.environ.get("OMP_NUM_THREADS", "0") or 0) or 16
+    threads = max(1, min(host_cpus, share))
     torch.set_num_threads(threads)
     freqs = oracle.build_freqs()
     S, B = w.chunk_tokens, w.rows
@@ -687,6 +745,7 @@ def cpu_baseline(args, w):
         "value": B * S / per_chunk,
         "unit": "tokens/s",
         "cores": threads,
+        "host_cpu_count": host_cpus,
         "kind": "port",
         "sample": (f"{n_chunks} steady-state chunks x {n_layers} layer(s) of {w.name} "
                    f"({dt:.1f} s), scaled to {w.layers} layers; torch {torch.__version__}"),
@@ -777,7 +836,10 @@ def main():
             "bytes_per_launch": w.append_bytes(with_q=False),
             "avg_launch_ms": g["append_ms"],
         },
-        "kernel_ms_per_layer": {"append": g["append_ms"], "attn": g["attn_ms"]},
+        "kernel_ms_per_layer": {
+            "append": g["append_ms"], "attn": g["attn_ms"],
+            "note": "from a second pass over the same steps in which every launch carries its own timing events "
+                    "(such dispatches run about 1 % longer): their sum can exceed ms_per_step / layers slightly"},
     }
     if g["fill_ms"] is not None:
         result["fill_phase_ms_per_chunk"] = [round(x, 4) for x in g["fill_ms"]]
@@ -793,6 +855,8 @@ def main():
         result["softmax_range"] = softmax_range_section(args, w)
     if args.torch_reference:
         result["torch_gpu_reference"] = torch_reference_section(args, w, g["ms_per_step"])
+    if not args.skip_mfma_ceiling:
+        result["mfma_ceiling"] = mfma_ceiling_section(achieved_tflops)
     if not args.skip_mfma_reference:
         ref = mfma_reference()
         ref["attention_vs_random"] = achieved_tflops / ref["random"]

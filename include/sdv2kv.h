@@ -120,9 +120,9 @@ typedef struct sdv2_append_params {
    * With both weights given, q_in and k_in are the raw projection outputs and
    *   x' = type_as(float(x) * rsqrt(mean_over_heads*128(float(x)^2) + norm_eps)) * weight
    * is what gets roped.  Weights have the tensors' dtype, heads * 128 elements.
-   * The mean is an fp32 sum in this kernel's order: against another summation
-   * order the normalised value can differ in its last fp32 bit, which shows as
-   * one storage-type ulp in about one element in 10^5.                        */
+   * The fp32 sum of squares is taken in the order of PyTorch's CPU sum kernel
+   * (vectors of 8 floats, 4 accumulators, blocks of 16), so the result is bit
+   * for bit what the two torch modules followed by the plain append store.     */
   const void* q_norm_weight;   /* device, or NULL (together with k_norm_weight) */
   const void* k_norm_weight;
   float norm_eps;

@@ -45,6 +45,30 @@ int sdv2_profile_time_next(int kernel, void* start, void* stop);
  * ---------------------------------------------------------------------- */
 int sdv2_copy_bytes(void* dst, const void* src, size_t bytes, void* stream);
 
+/* ------------------------------------------------------------------------
+ * What the GPU sustains on the attention kernel's own instruction streams.
+ * One launch of a kernel that runs the attention loop's matrix instructions
+ * on the caller's random operands, one workgroup per CU, `iterations` times
+ * three 64-key tiles, with parts of the loop taken away by `mode`; *flops
+ * receives the floating-point operations of the launch (32768 per MFMA).
+ * The caller times the launch (events on `stream`).  `operands` is device
+ * memory of at least sdv2_profile_mfma_stream_bytes() bytes, 256-byte aligned,
+ * filled with bf16 values (random for the realistic case: the rate a chip
+ * holds under matrix load depends on how much the operands toggle); only its
+ * last 512 KB are written, if ever.  Nothing is computed that anybody reads.
+ * ---------------------------------------------------------------------- */
+typedef enum sdv2_stream_mode {
+  SDV2_STREAM_REGISTERS = 0,      /* MFMAs alone, operands resident in registers               */
+  SDV2_STREAM_LDS_32_ROWS = 1,    /* + LDS fragment reads as the attention kernel makes them:
+                                     8 waves x 32 query rows, 1.5 reads per MFMA               */
+  SDV2_STREAM_LDS_64_ROWS = 2,    /* the same with 4 waves x 64 query rows: 0.75 reads per MFMA */
+  SDV2_STREAM_ATTENTION_MIX = 3   /* mode 1 + the softmax instructions between the MFMAs + the
+                                     global->LDS tile transfers and the barrier per tile       */
+} sdv2_stream_mode;
+size_t sdv2_profile_mfma_stream_bytes(void);
+int sdv2_profile_mfma_stream(int mode, const void* operands, size_t operand_bytes, int32_t iterations,
+                             void* stream, double* flops);
+
 #ifdef __cplusplus
 }
 #endif

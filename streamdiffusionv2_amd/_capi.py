@@ -29,6 +29,7 @@ DTYPE_BF16 = 0
 DTYPE_F32 = 1
 
 KERNEL_APPEND, KERNEL_ATTENTION, KERNEL_RELAYOUT, KERNEL_SINK, KERNEL_COPY = range(5)
+STREAM_REGISTERS, STREAM_LDS_32_ROWS, STREAM_LDS_64_ROWS, STREAM_ATTENTION_MIX = range(4)
 
 # every symbol include/sdv2kv.h and include/sdv2kv_profile.h declare
 EXPORTED_SYMBOLS = (
@@ -48,6 +49,8 @@ EXPORTED_SYMBOLS = (
     "sdv2_event_elapsed_ms",
     "sdv2_profile_time_next",
     "sdv2_copy_bytes",
+    "sdv2_profile_mfma_stream_bytes",
+    "sdv2_profile_mfma_stream",
 )
 
 
@@ -198,6 +201,11 @@ def lib() -> C.CDLL:
     handle.sdv2_profile_time_next.argtypes = [C.c_int, C.c_void_p, C.c_void_p]
     handle.sdv2_copy_bytes.restype = C.c_int
     handle.sdv2_copy_bytes.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+    handle.sdv2_profile_mfma_stream_bytes.restype = C.c_size_t
+    handle.sdv2_profile_mfma_stream_bytes.argtypes = []
+    handle.sdv2_profile_mfma_stream.restype = C.c_int
+    handle.sdv2_profile_mfma_stream.argtypes = [C.c_int, C.c_void_p, C.c_size_t, C.c_int32, C.c_void_p,
+                                                C.POINTER(C.c_double)]
     if handle.sdv2_abi_version() != ABI_VERSION:
         raise ImportError(
             f"{LIB_PATH} has ABI version {handle.sdv2_abi_version()}, expected {ABI_VERSION}: rebuild it"

@@ -153,6 +153,10 @@ class RingKVPath:
 
     # what the pinned decision words hold from the launch until the kernel has written them
     _NOT_YET = -(2 ** 31)
+    # How often (all paths of the process) a reader found the words still preset
+    # and had to wait for the stream: zero in a stream whose layers are called
+    # once per model pass; benchmarks print it.
+    decision_waits = 0
 
     def _decision_buffers(self, rows: int, dev):
         """Per path: the device slot override the decision kernel writes and
@@ -172,6 +176,7 @@ class RingKVPath:
         a reader that comes before they have arrived waits for the stream."""
         refresh = host.tolist()
         if self._NOT_YET in refresh:
+            RingKVPath.decision_waits += 1
             stream.synchronize()
             refresh = host.tolist()
             if self._NOT_YET in refresh:
@@ -191,11 +196,17 @@ class RingKVPath:
         self._sink_sums = None
 
     def _kept_sink_sums(self, kv_cache, rows: int, heads: int):
+        """The kept sums for this cache, all stale when anything says they may
+        not describe it: another dict (also a fresh one that got the old one's
+        memory back: the dict carries the token, not the address), other
+        tensors, another shape or sink size, contents changed from outside."""
         key = (kv_cache["k"].data_ptr(), kv_cache["v"].data_ptr(), tuple(kv_cache["k"].shape), self.sink_size,
                ring.contents_generation(kv_cache))
         kept = self._sink_sums
-        if kept is None or kept["key"] != key or len(kept["stale"]) != rows:
-            kept = dict(key=key, stale=[(1 << self.sink_size) - 1] * rows,
+        if kept is None or kept["key"] != key or len(kept["stale"]) != rows \
+                or kept["owner"] is not ring.sink_sums_owner(kv_cache):
+            kept = dict(key=key, owner=ring.sink_sums_owner(kv_cache, create=True),
+                        stale=[(1 << self.sink_size) - 1] * rows,
                         sums=ops.new_sink_frame_sums(rows, heads, self.sink_size, kv_cache["k"].device))
             self._sink_sums = kept
         return kept
@@ -204,7 +215,8 @@ class RingKVPath:
         """A call that did not run the check wrote plan.dst_start: the kept sums
         of the sink frames it touched are stale."""
         kept = self._sink_sums
-        if kept is None or kept["key"][0] != kv_cache["k"].data_ptr():
+        if kept is None or kept["key"][0] != kv_cache["k"].data_ptr() \
+                or kept["owner"] is not ring.sink_sums_owner(kv_cache):
             return
         for i, dst in enumerate(plan.dst_start[:len(kept["stale"])]):
             for frame in range(dst // frame_tokens, min(self.sink_size, (dst + tokens - 1) // frame_tokens + 1)):
@@ -285,6 +297,7 @@ class RingKVPath:
                 # reduction on the device, whose decision goes straight to the
                 # append below and, written into pinned memory by the kernel, to the host
                 override, host = self._decision_buffers(rows, q.device)
+                assert self._pending is None, "the last decision must be settled before its words are preset again"
                 host.fill_(self._NOT_YET)
                 kept = self._kept_sink_sums(kv_cache, rows, q.shape[2])
                 extra = {}
@@ -352,6 +365,9 @@ class RingKVPath:
                 # before a later call presets them again
                 self._pending["stream"].synchronize()
             self._evict_idx, self._pending, self._sink_sums = undo[0], None, None
+            # a launch that was refused started nothing; one that failed on the device may have left
+            # ticket words of this stream's workspaces non-zero, which every later call would trip over
+            ops.reset_workspace_tickets(q.device)
             if undo[1] is not None:
                 kv_cache["current_step"] = undo[1]
             ring.forget_index_mirror(kv_cache)        # the device tensors are authoritative again

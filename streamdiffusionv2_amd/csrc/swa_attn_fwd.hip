@@ -200,6 +200,22 @@ __device__ __forceinline__ u32x2 lds_read_tr16_b64(uint32_t addr) {
   asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(kOffset));
   return r;
 }
+// The same reads for the exact pass, which is not pipelined: the value is
+// waited for inside the statement and handed to compiler-generated MFMAs.
+// (Absolute per-lane addresses as in the fast pass: taking them relative to
+// the LDS base would keep a second copy of all sixteen alive across the
+// streaming loop.)
+__device__ __forceinline__ bf16x8 lds_read_b128_now(uint32_t addr) {
+  u32x4 r;
+  asm volatile("ds_read_b128 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(r) : "v"(addr) : "memory");
+  return __builtin_bit_cast(bf16x8, r);
+}
+__device__ __forceinline__ bf16x8 lds_read_tr16_b64x2_now(uint32_t addr_lo, uint32_t addr_hi) {
+  u32x2 lo, hi;
+  asm volatile("ds_read_b64_tr_b16 %0, %2\n\tds_read_b64_tr_b16 %1, %3\n\ts_waitcnt lgkmcnt(0)"
+               : "=&v"(lo), "=&v"(hi) : "v"(addr_lo), "v"(addr_hi) : "memory");
+  return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3));
+}
 // Optimisation passes may sink pure arithmetic down to its first use, which
 // here is a whole pipeline slot later.  Passing a value through an empty
 // volatile asm fixes the point by which it has to be computed.
@@ -527,8 +543,7 @@ __device__ __forceinline__ void exact_pass(const LaneConst& c, const bf16x8 (&qf
         for (int i = 0; i < 16; ++i) sacc[kb][i] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) {
-          const bf16x8 kf = *reinterpret_cast<__attribute__((address_space(3))) const bf16x8*>(
-              lds + (c.k_addr[ks] - lds_addr0) + kb_off + kb * 32 * 256);
+          const bf16x8 kf = lds_read_b128_now(c.k_addr[ks] + (uint32_t)(kb_off + kb * 32 * 256));
           sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc[kb], 0, 0, 0);
         }
         if (key0 + kb * 32 + 32 > seq || (key0 + kb * 32 + 32 > c.wg_m_lo && key0 + kb * 32 < c.m_hi))
@@ -568,13 +583,9 @@ __device__ __forceinline__ void exact_pass(const LaneConst& c, const bf16x8 (&qf
         for (int i = 0; i < 16; ++i) oacc[db][i] *= alpha;
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(
-              lds + (c.v_addr[db][0] - lds_addr0) + vb_off + kk * 16 * 256));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)(
-              lds + (c.v_addr[db][1] - lds_addr0) + vb_off + kk * 16 * 256));
-          const s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-          oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, both), pf[kk >> 1][kk & 1],
-                                                              oacc[db], 0, 0, 0);
+          const bf16x8 vf = lds_read_tr16_b64x2_now(c.v_addr[db][0] + (uint32_t)(vb_off + kk * 16 * 256),
+                                                    c.v_addr[db][1] + (uint32_t)(vb_off + kk * 16 * 256));
+          oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kk >> 1][kk & 1], oacc[db], 0, 0, 0);
         }
       }
     }
@@ -1152,6 +1163,8 @@ extern "C" int sdv2_swa_attn_fwd_static(const sdv2_attn_params* p) {
   if (!p) return SDV2_ERR_INVALID_ARG;
   if (p->rows <= 0 || p->q_tokens <= 0 || p->heads <= 0 || p->max_seq_len < 0)
     return attn_fwd(p, nullptr, 0);                       // nothing to split: same answers as the plain entry point
+  if (p->dtype == SDV2_F32) return attn_fwd(p, nullptr, 0);   // fp32 walks one key range: no scratch, whatever num_splits says
+  if (p->num_splits > 64) return SDV2_ERR_INVALID_ARG;        // as the plain entry point answers
   const int splits = p->num_splits > 0 ? p->num_splits
                                        : sdv2_swa_attn_default_splits(p->rows, p->q_tokens, p->heads, p->max_seq_len);
   if (splits <= 1) return attn_fwd(p, nullptr, 0);

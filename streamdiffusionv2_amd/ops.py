@@ -259,10 +259,30 @@ def causal_rope_apply(x: torch.Tensor, grid_sizes, freqs: torch.Tensor, start_fr
 _WORKSPACES: dict = {}
 
 
+TICKET_BYTES = 65536          # head of an attention workspace (256 bytes for a sink-similarity one)
+
+
 def new_workspace(dev: torch.device, nbytes: int) -> torch.Tensor:
     """A split-KV workspace as the library wants it: zero-filled once (its
-    ticket words start at zero and every call leaves them there)."""
-    return torch.zeros(max(nbytes, 1), dtype=torch.uint8, device=dev)
+    ticket words start at zero and every call leaves them there).  Only
+    buffers made here are accepted as ``workspace=``: a ticket word that does
+    not start at zero makes a split call combine early or never, silently."""
+    ws = torch.zeros(max(nbytes, 1), dtype=torch.uint8, device=dev)
+    ws._sdv2_workspace = True
+    return ws
+
+
+def reset_workspace_tickets(dev: torch.device) -> None:
+    """Zero the ticket words of this stream's workspaces again.  Every call
+    that completes leaves them at zero; after a launch that failed on the
+    device they may not be."""
+    if dev.type != "cuda" or not (_WORKSPACES or _SIM_WORKSPACES):
+        return
+    key = (dev, _stream_ptr(dev))
+    for pool in (_WORKSPACES, _SIM_WORKSPACES):
+        ws = pool.get(key)
+        if ws is not None:
+            ws[:TICKET_BYTES].zero_()
 
 
 def _workspace(dev: torch.device, nbytes: int, pool: Optional[dict] = None) -> torch.Tensor:
@@ -355,6 +375,8 @@ def swa_attention(
     elif num_splits <= 0:
         num_splits = lib.sdv2_swa_attn_default_splits(rows, q_tokens, heads, max_seq_len)
     need = 0 if static_scratch else lib.sdv2_swa_attn_workspace_bytes(rows, q_tokens, heads, max_seq_len, num_splits)
+    if workspace is not None and not getattr(workspace, "_sdv2_workspace", False):
+        raise RuntimeError("workspace= takes a buffer made by ops.new_workspace() (zero-filled ticket words)")
     if need and (workspace is None or workspace.numel() * workspace.element_size() < need):
         workspace = _workspace(dev, need)
 

@@ -28,6 +28,7 @@ import torch
 HEAD_DIM = 128
 _MIRROR_KEY = "_sdv2_host_index_mirror"
 _GENERATION_KEY = "_sdv2_contents_generation"
+_SINK_OWNER_KEY = "_sdv2_sink_sums_owner"
 
 
 def tensor_version(t: torch.Tensor) -> Optional[int]:
@@ -87,6 +88,7 @@ def replicate_for_stream_batch(kv_cache: List[dict], batch_size: int) -> None:
         entry["global_end_index"] = entry["global_end_index"].repeat(batch_size)
         entry["local_end_index"] = entry["local_end_index"].repeat(batch_size)
         entry.pop(_MIRROR_KEY, None)
+        entry.pop(_SINK_OWNER_KEY, None)
 
 
 def new_crossattn_cache(num_layers: int, batch_size: int, heads: int, dtype=torch.bfloat16, device="cuda",
@@ -167,6 +169,18 @@ def contents_changed(kv_cache: dict) -> None:
 
 def contents_generation(kv_cache: dict) -> int:
     return kv_cache.get(_GENERATION_KEY, 0)
+
+
+def sink_sums_owner(kv_cache: dict, create: bool = False):
+    """The token that ties a path's kept sink-frame sums to THIS cache dict.
+    Addresses do not identify a cache: a cache allocated after another was
+    dropped usually gets the same memory back, while its contents (zeros) are
+    new.  A dict that never went through a check carries no token."""
+    token = kv_cache.get(_SINK_OWNER_KEY)
+    if token is None and create:
+        token = object()
+        kv_cache[_SINK_OWNER_KEY] = token
+    return token
 
 
 @dataclass

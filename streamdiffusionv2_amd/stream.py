@@ -128,6 +128,8 @@ class KVStreamPipeline:
         for p in self.generator.paths:
             p.sink_size = self.num_sink_tokens
             p.adapt_sink_thr = self.adapt_sink_threshold
+            if hasattr(p, "forget_sink_sums"):
+                p.forget_sink_sums()      # a new cache: nothing a path summed before describes it
         self.kv_cache1 = self._cache_factory(
             self.num_transformer_blocks, batch_size, self.kv_cache_length, self.num_heads,
             len(self.denoising_step_list), dtype=dtype, device=device)
@@ -137,6 +139,9 @@ class KVStreamPipeline:
         attention modules and are NOT reset, as in the reference."""
         self.kv_cache1 = None
         self.hidden_states = None
+        for p in self.generator.paths:
+            if hasattr(p, "forget_sink_sums"):
+                p.forget_sink_sums()
 
     # -- causal_stream_inference.py:124-255 --------------------------------
     def prepare(self, noise: torch.Tensor, current_start: int = 0, current_end: Optional[int] = None,

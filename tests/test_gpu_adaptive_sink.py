@@ -257,6 +257,75 @@ def test_stream_with_refresh(gpu_device, seed, rows, look_every_call):
         assert err.max().item() <= 2e-2 * unit and err.mean().item() <= 2e-3 * unit, call
 
 
+def _oracle_sessions(seed, sessions, calls, heads=2, sink=3, cache_frames=6):
+    """One oracle layer run through several streams, each on a cache of its own
+    that starts out all zero; the layer (and its eviction queue, which the
+    reference does not reset either) lives on."""
+    gen = torch.Generator().manual_seed(seed)
+    basis = torch.randn(3, heads * 128, generator=gen)
+    freqs = oracle.build_freqs()
+    layer = oracle.RingAttentionOracle(sink_size=sink, adapt_sink_thr=THR)
+    out, sims = [], []
+    for _ in range(sessions):
+        cache = oracle.new_kv_cache(1, 1, cache_frames * FT, heads, 1, dtype=torch.bfloat16)[0]
+        record = []
+        for call in range(calls):
+            if call % 4 == 0:
+                scene = torch.randn(3, generator=gen)
+            q, k, v = directed_chunk(gen, 1, heads, torch.bfloat16, basis, scene)
+            starts = [call * FT]
+            _, roped_q, seq = layer.step(q, k, v, [GRID], freqs, cache, starts, with_attention=False)
+            sims.extend(layer.last_sims)
+            record.append(dict(q=q, k=k, v=v, starts=starts, seq=seq, writes=list(layer.last_writes),
+                               queue=[list(x) for x in layer.evict_idx], sims=[x.clone() for x in layer.last_sims],
+                               cache_k=cache["k"].clone(), cache_v=cache["v"].clone()))
+        out.append(record)
+    return out, sims
+
+
+def test_two_session_recipe_has_clear_margins_on_the_oracle():
+    sessions, sims = _oracle_sessions(10, 2, 9)
+    assert oracle_margins_ok(sims), [x.tolist() for x in sims]
+    # the second stream starts on zeros: its first checks see cosine 0 and refresh, whatever the first stream held
+    assert all(x.min().item() == 0.0 for x in sessions[1][0]["sims"])
+
+
+@pytest.mark.gpu
+def test_a_fresh_cache_at_the_old_address_is_summed_afresh(gpu_device):
+    """The kept means of the sink frames belong to one cache dict.  A stream
+    that is reset and started again (streamv2v/inference.py:161-171, then
+    causal_stream_inference.py:87-107) gets a new all-zero cache, usually in
+    the very memory the old one had, while the path object lives on: the first
+    checks of the new stream must compare against zeros, as the reference
+    does, not against what the old stream's sink frames held."""
+    from streamdiffusionv2_amd import ring, rope
+    from streamdiffusionv2_amd.attention import RingKVPath
+
+    heads, sink, cache_frames = 2, 3, 6
+    sessions, sims = _oracle_sessions(10, 2, 9)
+    assert oracle_margins_ok(sims)
+    freqs = rope.build_freqs()
+    path = RingKVPath(sink_size=sink, adapt_sink_thr=THR)
+    old_address = None
+    for number, record in enumerate(sessions):
+        cache = ring.new_kv_cache(1, 1, cache_frames * FT, heads, 1, device=gpu_device)[0]
+        print(f"session {number}: cache at {cache['k'].data_ptr():#x} (the last one at {old_address})", flush=True)
+        for call, rec in enumerate(record):
+            path.attend(rec["q"].to(gpu_device), rec["k"].to(gpu_device), rec["v"].to(gpu_device),
+                        torch.tensor([GRID]), freqs, cache, rec["starts"])
+            torch.cuda.synchronize()
+            want_refresh = [int(x.argmin()) if x.min().item() < THR else -1 for x in rec["sims"]]
+            assert path.last_refresh == want_refresh, (number, call)
+            assert path.evict_idx == rec["queue"], (number, call)
+            assert [(a, a + FT) for a in path.last_plan.dst_start] == rec["writes"], (number, call)
+            assert cache["local_end_index"].tolist() == rec["seq"], (number, call)
+            for name in ("k", "v"):
+                assert torch.equal(cache[name].cpu().view(torch.int16), rec["cache_" + name].view(torch.int16)), \
+                    (number, call, name)
+        old_address = hex(cache["k"].data_ptr())
+        del cache
+
+
 # --------------------------------------------------------------------------
 # The shipped shape: 480p latent frames of 30 x 52 = 1560 tokens, sink 3,
 # threshold 0.2 (configs/wan_causal_dmd_v2v.yaml:53-56), 12 heads (Wan 1.3B)

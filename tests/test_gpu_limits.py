@@ -117,3 +117,48 @@ def test_a_failed_call_leaves_the_ring_state_where_it_was(gpu_device):
         assert torch.equal(a, b)
     assert path.evict_idx == twin_path.evict_idx
     assert torch.equal(cache["k"], twin["k"]) and torch.equal(cache["v"], twin["v"])
+
+
+def test_a_split_call_after_a_refused_one_is_still_right(gpu_device):
+    """A call the library refuses (status < 0) launches nothing and leaves the
+    ticket words of the workspace at zero; the wrapper zeroes them again after
+    any failed layer call.  Either way the next split call combines its key
+    ranges as if nothing had happened."""
+    from streamdiffusionv2_amd import ops
+
+    torch.manual_seed(3)
+    rows, S, H, L, sp = 1, 300, 3, 2500, 4
+    q = torch.randn(rows, S, H, 128).bfloat16()
+    k = torch.randn(rows, L, H, 128).bfloat16()
+    v = torch.randn(rows, L, H, 128).bfloat16()
+    qd, kd, vd = q.to(gpu_device), k.to(gpu_device), v.to(gpu_device)
+    want = oracle.attention_fp32_reference(q, k, v, [L] * rows)
+    first = ops.swa_attention(qd, kd, vd, None, num_splits=sp)
+    with pytest.raises(RuntimeError):                    # refused: misaligned output pointer
+        ops.swa_attention(qd, kd, vd, None, num_splits=sp, out=torch.empty(rows, S, H, 129, dtype=torch.bfloat16,
+                                                                           device=gpu_device)[..., 1:])
+    with pytest.raises(RuntimeError):                    # refused: more key ranges than the library takes
+        ops.swa_attention(qd, kd, vd, None, num_splits=65)
+    again = ops.swa_attention(qd, kd, vd, None, num_splits=sp)
+    ops.reset_workspace_tickets(gpu_device)              # what a failed layer call does on its way out
+    third = ops.swa_attention(qd, kd, vd, None, num_splits=sp)
+    torch.cuda.synchronize()
+    for got in (first, again, third):
+        assert torch.equal(got, first)
+        err = (got.float().cpu() - want).abs()
+        assert err.max().item() <= 2e-2 and err.mean().item() <= 2e-3
+
+
+def test_only_zero_filled_workspaces_are_accepted(gpu_device):
+    """A caller-owned workspace must come from ops.new_workspace: a ticket word
+    that does not start at zero would make a split call combine early or never,
+    with no error to show for it."""
+    from streamdiffusionv2_amd import _capi, ops
+
+    q = torch.zeros(1, 64, 1, 128, dtype=torch.bfloat16, device=gpu_device)
+    kv = torch.zeros(1, 2048, 1, 128, dtype=torch.bfloat16, device=gpu_device)
+    need = _capi.lib().sdv2_swa_attn_workspace_bytes(1, 64, 1, 2048, 2)
+    with pytest.raises(RuntimeError):
+        ops.swa_attention(q, kv, kv, None, num_splits=2, workspace=torch.empty(need, dtype=torch.uint8, device=gpu_device))
+    ops.swa_attention(q, kv, kv, None, num_splits=2, workspace=ops.new_workspace(gpu_device, need))
+    torch.cuda.synchronize()

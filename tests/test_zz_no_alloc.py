@@ -90,6 +90,22 @@ def test_static_entry_point_refuses_more_than_it_holds(gpu_device):
     _capi.check(lib.sdv2_swa_attn_fwd_static(C.byref(_attn_params(q, kc, kc, out, None, 1))), "static, unsplit")
     torch.cuda.synchronize()
     assert bool((out == 0.0).all())
+    # more key ranges than the library ever takes: the plain entry point's answer, not a scratch complaint
+    too_many = _attn_params(q, kc, kc, out, None, 65)
+    assert lib.sdv2_swa_attn_fwd_static(C.byref(too_many)) == _capi.SDV2_ERR_INVALID_ARG
+    ws = torch.zeros(8, dtype=torch.uint8, device=gpu_device)
+    too_many.workspace, too_many.workspace_bytes = ws.data_ptr(), ws.numel()
+    assert lib.sdv2_swa_attn_fwd(C.byref(too_many)) == _capi.SDV2_ERR_INVALID_ARG
+    # fp32 tensors walk one key range and need no scratch, whatever the shape and num_splits say
+    qf = torch.zeros(4, 4680, 12, 128, dtype=torch.float32, device=gpu_device)
+    kf = torch.zeros(4, 640, 12, 128, dtype=torch.float32, device=gpu_device)
+    of = torch.full_like(qf, 3.0)
+    fp32 = _attn_params(qf, kf, kf, of, None, 64)
+    fp32.dtype = _capi.DTYPE_F32
+    assert lib.sdv2_swa_attn_workspace_bytes(4, 4680, 12, 640, 64) > _capi.STATIC_SCRATCH_BYTES   # were it bf16
+    _capi.check(lib.sdv2_swa_attn_fwd_static(C.byref(fp32)), "static, fp32")
+    torch.cuda.synchronize()
+    assert bool((of == 0.0).all())
 
 
 def test_static_entry_point_at_the_wan_shapes(gpu_device):
