@@ -147,6 +147,8 @@ def parse_args():
     ap.add_argument("--softmax-range", action="store_true",
                     help="also time the attention launch with the queries scaled up until rows leave the range the fast "
                          "softmax covers and waves redo their block with the running-maximum recurrence")
+    ap.add_argument("--skip-module-path", action="store_true",
+                    help="do not time the path as a module call drives it (fused q / k norm; shipped sink settings)")
     ap.add_argument("--skip-mfma-ceiling", action="store_true",
                     help="do not run the library's own MFMA / LDS / softmax instruction streams (what this box sustains "
                          "on the attention kernel's instruction mix)")
@@ -338,14 +340,16 @@ def mfma_ceiling_section(achieved_tflops):
     stream = torch.cuda.current_stream(dev).cuda_stream
     flops = C.c_double()
     names = (("mfma_only_registers", _capi.STREAM_REGISTERS), ("lds_reads_32_rows_per_wave", _capi.STREAM_LDS_32_ROWS),
-             ("lds_reads_64_rows_per_wave", _capi.STREAM_LDS_64_ROWS), ("attention_loop_mix", _capi.STREAM_ATTENTION_MIX))
+             ("lds_reads_64_rows_per_wave", _capi.STREAM_LDS_64_ROWS), ("attention_loop_mix", _capi.STREAM_ATTENTION_MIX),
+             ("attention_loop_mix_64_rows_per_wave", _capi.STREAM_ATTENTION_MIX_64_ROWS))
     for kind in ("random", "zeros"):
         if kind == "random":
             buf = (torch.randn(nbytes // 2, device=dev) * 0.3).bfloat16()
         else:
             buf = torch.zeros(nbytes // 2, device=dev, dtype=torch.bfloat16)
         for name, mode in names:
-            if kind == "zeros" and mode not in (_capi.STREAM_REGISTERS, _capi.STREAM_ATTENTION_MIX):
+            if kind == "zeros" and mode not in (_capi.STREAM_REGISTERS, _capi.STREAM_ATTENTION_MIX,
+                                                _capi.STREAM_ATTENTION_MIX_64_ROWS):
                 continue
 
             def launch():
@@ -366,6 +370,177 @@ def mfma_ceiling_section(achieved_tflops):
         del buf
     out["attention_kernel_vs_attention_loop_mix"] = achieved_tflops / out["attention_loop_mix"]
     out["frac_of_peak_attention_loop_mix"] = out["attention_loop_mix"] / PEAK_BF16_TFLOPS
+    return out
+
+
+def module_path_section(args, w, headline_ms):
+    """What a model call executes, beside the headline (which times the path on
+    q / k that are already normalised, with the sink check off):
+
+    * ``fused_norm``: the path as CausalWanSelfAttention.forward drives it by
+      default - raw q / k projections in, their RMSNorm folded into the append
+      (causal_model.py:212-218), the query normalised and rotated inside the
+      attention kernel;
+    * ``shipped_config``: the same with the shipped v2v settings, sink 3 and
+      adaptive threshold 0.2 (configs/wan_causal_dmd_v2v.yaml:53-56).  The
+      inputs carry a scene direction that changes every eighth chunk, so the
+      refresh check keeps the sink frames most of the time and replaces them,
+      one per chunk, after a cut;
+    * ``module_forward``: whole forward() calls, with the four projection GEMMs
+      (vendor library) around the path.
+    Steady state, one chunk per step through every layer."""
+    from streamdiffusionv2_amd import ring, workloads
+    from streamdiffusionv2_amd.attention import CausalWanSelfAttention, RingKVPath
+
+    dev = torch.device("cuda:0")
+    freqs = build_freqs()
+    S, H, B = w.chunk_tokens, w.heads, w.rows
+    grid = torch.tensor([list(w.grid)] * B, dtype=torch.long)
+    max_chunk = (1024 - w.grid[0]) // w.grid[0]
+    eps = 1e-6
+    gen = torch.Generator(device=dev).manual_seed(9)
+    # raw projection outputs: a few times the unit scale, as before a norm
+    qkv = [tuple((t.float() * 3.0).to(w.dtype).to(dev) for t in workloads.make_qkv(w, 0, layer)) for layer in range(w.layers)]
+    wq = [(torch.rand(H * 128, device=dev, generator=gen) + 0.5).to(w.dtype) for _ in range(w.layers)]
+    wk = [(torch.rand(H * 128, device=dev, generator=gen) + 0.5).to(w.dtype) for _ in range(w.layers)]
+    fill = w.cache_tokens // S + B + 1
+    out = {}
+
+    def run(paths, caches, inputs_for, steps, per_step=None):
+        state = {"call": 0}
+
+        def step():
+            call = state["call"]
+            starts = [min(c, max_chunk) * S for c in workloads.row_chunks(w, call)]
+            for layer in range(w.layers):
+                q, k, v = inputs_for(call, layer)
+                paths[layer].attend(q, k, v, grid, freqs, caches[layer], starts, qk_norm=(wq[layer], wk[layer], eps))
+            state["call"] += 1
+
+        for _ in range(fill + args.warmup):
+            step()
+        torch.cuda.synchronize()
+        waits = RingKVPath.decision_waits
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+        state["waits"] = RingKVPath.decision_waits - waits
+        if per_step is not None:
+            # the same stream a little further, every step timed and looked at on its own
+            for _ in range(steps):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                step()
+                e1.record()
+                torch.cuda.synchronize()
+                refreshed = sum(1 for p in paths if p.last_refresh and p.last_refresh[0] >= 0)
+                per_step.append((e0.elapsed_time(e1), refreshed))
+        return ms, state["waits"]
+
+    def fresh(sink, thr):
+        caches = ring.new_kv_cache(w.layers, 1, w.cache_tokens, H, total_steps=1, dtype=w.dtype, device=dev)
+        if B > 1:
+            ring.replicate_for_stream_batch(caches, B)
+        return [RingKVPath(sink_size=sink, adapt_sink_thr=thr) for _ in range(w.layers)], caches
+
+    paths, caches = fresh(w.sink_size, -1)
+    ms, _ = run(paths, caches, lambda call, layer: qkv[layer], args.steps)
+    out["fused_norm"] = {"ms_per_step": ms, "vs_headline": ms / headline_ms,
+                         "what": "attend() on raw q / k with the q / k RMSNorm inside the kernels, sink check off"}
+    # the two kernels' own durations on this path (timing events in each dispatch), a few more steps of the same stream
+    from streamdiffusionv2_amd import ops
+    table = ops.device_freqs(freqs, dev)
+    timers = []
+    call = fill + args.warmup + args.steps
+    for _ in range(max(2, args.steps // 4)):
+        starts = [min(c, max_chunk) * S for c in workloads.row_chunks(w, call)]
+        for layer in range(w.layers):
+            q, k, v = qkv[layer]
+            norm = (wq[layer], wk[layer], eps)
+            plan = ring.plan_append(caches[layer], paths[layer].evict_idx, starts, S, w.frame_tokens, paths[layer].sink_size)
+            launcher = paths[layer]._layer_launcher(q, k, v, caches[layer], table, w.grid, norm)
+            launcher.patch(q, k, v, [c // w.frame_tokens for c in starts], plan, None)
+            t = (ops.KernelTimer(), ops.KernelTimer())
+            launcher.set_timers(*t)
+            launcher.run_append()
+            launcher.run_attention()
+            launcher.set_timers()
+            timers.append(t)
+        call += 1
+    torch.cuda.synchronize()
+    out["fused_norm"]["kernel_ms_per_layer"] = {
+        "append_with_norm": sum(t[0].elapsed_ms() for t in timers) / len(timers),
+        "attention_with_q_norm": sum(t[1].elapsed_ms() for t in timers) / len(timers)}
+    out["fused_norm"]["append_bytes"] = w.append_bytes(with_q=True) * 5 // 6      # read q, k, v; write k', v
+    out["fused_norm"]["append_GBps"] = out["fused_norm"]["append_bytes"] / (
+        out["fused_norm"]["kernel_ms_per_layer"]["append_with_norm"] * 1e-3) / 1e9
+    for t in timers:
+        for x in t:
+            x.close()
+    del paths, caches
+
+    if S == w.frame_tokens and B == 1:
+        # two scenes: a direction common to all tokens of a chunk, added to k and v
+        scenes = []
+        for s_ in range(2):
+            per_layer = []
+            for layer in range(w.layers):
+                q, k, v = qkv[layer]
+                dk = torch.randn(1, 1, H, 128, device=dev, generator=gen) * 3.0 * w.input_scale
+                dv = torch.randn(1, 1, H, 128, device=dev, generator=gen) * 3.0 * w.input_scale
+                per_layer.append((q, (k.float() + dk).to(w.dtype), (v.float() + dv).to(w.dtype)))
+            scenes.append(per_layer)
+        period = 8
+        paths, caches = fresh(3, 0.2)
+        per_step = []
+        ms, waits = run(paths, caches, lambda call, layer: scenes[(call // period) % 2][layer], max(args.steps, 2 * period),
+                        per_step)
+        quiet = [t for t, r in per_step if r == 0]
+        busy = [t for t, r in per_step if r > 0]
+        out["shipped_config"] = {
+            "sink_size": 3, "adapt_sink_thr": 0.2, "ms_per_step": ms, "vs_headline": ms / headline_ms,
+            "steps_timed": max(args.steps, 2 * period), "scene_cut_every_chunks": period,
+            "steps_with_a_refresh": len(busy), "steps_without": len(quiet),
+            "layers_refreshing_in_such_a_step": (sum(r for _, r in per_step if r > 0) / len(busy)) if busy else 0,
+            "ms_per_step_refreshing": (sum(busy) / len(busy)) if busy else None,
+            "ms_per_step_not_refreshing": (sum(quiet) / len(quiet)) if quiet else None,
+            # times the host found a decision not yet written and had to wait for the stream (timed pass)
+            "host_waits_for_a_decision": waits,
+            "what": "fused norm + adaptive sink refresh (one more launch per layer), scene cut every 8th chunk"}
+        del paths, caches, scenes
+
+    # whole module calls: q / k / v / o projections around the path
+    dim = H * 128
+    layers = min(w.layers, 8)
+    mods = [CausalWanSelfAttention(dim, H).to(dev).to(w.dtype) for _ in range(layers)]
+    for m in mods:
+        m.sink_size = w.sink_size
+    caches = ring.new_kv_cache(layers, 1, w.cache_tokens, H, total_steps=1, dtype=w.dtype, device=dev)
+    if B > 1:
+        ring.replicate_for_stream_batch(caches, B)
+    x = (torch.randn(B, S, dim, device=dev, generator=gen)).to(w.dtype)
+    state = {"call": 0}
+
+    def module_step():
+        starts = torch.tensor([min(c, max_chunk) * S for c in workloads.row_chunks(w, state["call"])])
+        for layer in range(layers):
+            mods[layer](x, None, grid, freqs, None, kv_cache=caches[layer], current_start=starts)
+        state["call"] += 1
+
+    with torch.no_grad():
+        for _ in range(fill + args.warmup):
+            module_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            module_step()
+        torch.cuda.synchronize()
+    per_layer = (time.perf_counter() - t0) * 1e3 / (args.steps * layers)
+    out["module_forward"] = {"ms_per_layer_call": per_layer, "ms_per_step": per_layer * w.layers, "layers_timed": layers,
+                             "what": "CausalWanSelfAttention.forward with its defaults: q / k / v / o projections "
+                                     "(vendor GEMMs) + the path; scaled to the layer count"}
     return out
 
 
@@ -417,16 +592,28 @@ def qk_norm_section(args, w):
         torch.cuda.synchronize()
         out[name] = e0.elapsed_time(e1) / n
     out["bytes_per_launch"] = w.append_bytes(with_q=True)
-    # the fused kernel's own duration (timing events in its dispatch)
+    # the fused kernel's own duration (timing events in its dispatch): as the operator returns the rotated
+    # query (read q, k, v; write q', k', v), and as the module path runs it (q is only read, for its sum of
+    # squares; the attention kernel normalises and rotates the raw q itself)
+    inv_rms = torch.empty(B, S, dtype=torch.float32, device=dev)
+
+    def fused_no_q_out(i):
+        q, k, v = qkv[i % layers]
+        c = caches[i % layers]
+        ops.kv_append_rope(q, k, v, c["k"], c["v"], table, w.grid, starts, dst, qk_norm=weights, q_inv_rms=inv_rms)
+
     timer = ops.KernelTimer()
-    kernel_ms = []
-    for i in range(n):
-        timer.arm(_capi.KERNEL_APPEND)
-        fused(i)
-        kernel_ms.append(timer.elapsed_ms())
+    for name, fn, moved in (("fused_kernel", fused, w.append_bytes(with_q=True)),
+                            ("fused_kernel_no_q_out", fused_no_q_out, w.append_bytes(with_q=True) * 5 // 6)):
+        kernel_ms = []
+        for i in range(n):
+            timer.arm(_capi.KERNEL_APPEND)
+            fn(i)
+            kernel_ms.append(timer.elapsed_ms())
+        out[name + "_ms"] = sum(kernel_ms) / len(kernel_ms)
+        out[name + "_bytes"] = moved
+        out[name + "_GBps"] = moved / (out[name + "_ms"] * 1e-3) / 1e9
     timer.close()
-    out["fused_kernel_ms"] = sum(kernel_ms) / len(kernel_ms)
-    out["fused_kernel_GBps"] = out["bytes_per_launch"] / (out["fused_kernel_ms"] * 1e-3) / 1e9
     out["note"] = ("fused_ms / torch_norms_plus_append_ms are host-inclusive per-call times (the torch path launches "
                    "about a dozen kernels per call); fused_kernel_ms is the kernel alone")
     # The consumer side (causal_model.py:387-389): the o projection reads the attention output in place.
@@ -812,7 +999,9 @@ def main():
             "workload": w.name,
             "layers": w.layers, "rows": w.rows, "heads": w.heads, "head_dim": 128,
             "chunk_tokens": w.chunk_tokens, "cache_tokens": w.cache_tokens,
-            "grid": list(w.grid), "kv_splits": g["splits"],
+            "grid": list(w.grid), "kv_splits": g["splits"] & 255,
+            # of each XCD's share of the (row, head) pairs, how many take one key range more
+            "kv_splits_one_more_on_pairs_per_xcd": g["splits"] >> 8,
         },
         "roofline": {
             "kernel": "swa_attn_fwd_kernel",
@@ -855,6 +1044,8 @@ def main():
         result["softmax_range"] = softmax_range_section(args, w)
     if args.torch_reference:
         result["torch_gpu_reference"] = torch_reference_section(args, w, g["ms_per_step"])
+    if not args.skip_module_path and not args.zero_inputs:
+        result["module_path"] = module_path_section(args, w, g["ms_per_step"])
     if not args.skip_mfma_ceiling:
         result["mfma_ceiling"] = mfma_ceiling_section(achieved_tflops)
     if not args.skip_mfma_reference:

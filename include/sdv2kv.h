@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SDV2KV_ABI_VERSION 10
+#define SDV2KV_ABI_VERSION 11
 #define SDV2_HEAD_DIM 128      /* causal_stream_inference.py:99-100 fixes 128 */
 #define SDV2_MAX_ROWS 16       /* rows (B) per sdv2_kv_append_rope call       */
 #define SDV2_MAX_SINK_FRAMES 16 /* sink frames per sdv2_sink_similarity call  */
@@ -131,6 +131,11 @@ typedef struct sdv2_append_params {
    * writes it, so that an adaptive sink refresh needs no host round trip
    * between the decision and the append.                                      */
   const int64_t* dst_start_override;
+  /* Optional, with the norm weights: device float [B * S] that receives
+   * rsqrt(mean(q^2) + norm_eps) of every query token.  q_out may then be NULL:
+   * no rotated query is written, and sdv2_swa_attn_fwd normalises and rotates
+   * the raw q itself (its q_norm_weight / q_inv_rms), to the same bits.       */
+  float* q_inv_rms;
 } sdv2_append_params;
 
 int sdv2_kv_append_rope(const sdv2_append_params* p);
@@ -172,7 +177,13 @@ typedef struct sdv2_attn_params {
   sdv2_stride3 q_stride, k_stride, v_stride, out_stride;
   int32_t rows, q_tokens, heads, head_dim;        /* B, S, H, 128              */
   int32_t max_seq_len;                            /* L = k_cache.shape[1]      */
-  int32_t num_splits;          /* 0 = choose from the shape                    */
+  int32_t num_splits;          /* key ranges per (row, head); 0 = choose from the
+                                * shape.  Bits 0-7: the count s (<= 64).  Bits 8-15
+                                * (optional, needs rows * heads divisible by 8): of
+                                * every eighth of the (row, head) list - one XCD's
+                                * share - that many pairs take s + 1 ranges instead,
+                                * which fills the last round of workgroups better.
+                                * sdv2_swa_attn_default_splits returns this form.  */
   float softmax_scale;         /* <= 0 selects 1/sqrt(head_dim)                */
   void* workspace;             /* device scratch, 256-byte aligned             */
   size_t workspace_bytes;
@@ -203,9 +214,17 @@ typedef struct sdv2_attn_params {
    * one key range (num_splits, workspace and rope_freqs must be unset: fp32
    * queries arrive rotated), strides in multiples of 4 elements.             */
   int32_t dtype;
+  /* Optional q RMSNorm inside the call (needs rope_freqs and SDV2_BF16): q is
+   * the raw q projection, q_norm_weight the norm's weight (device, bf16,
+   * heads * 128 elements, 16-byte aligned) and q_inv_rms what
+   * sdv2_kv_append_rope stored (device float [B * S]).  Every element is
+   * normalised (x * inv_rms rounded to bf16, times weight rounded to bf16, as
+   * WanRMSNorm rounds, wan_base/modules/model.py:77-86) and then rotated.      */
+  const void* q_norm_weight;
+  const float* q_inv_rms;
 } sdv2_attn_params;
 
-/* number of key-range splits the library would pick for this shape */
+/* the key-range split plan the library would pick for this shape, as num_splits carries it */
 int sdv2_swa_attn_default_splits(int32_t rows, int32_t q_tokens, int32_t heads, int32_t max_seq_len);
 /* bytes of workspace needed for `num_splits` (0 = default); 0 when unsplit */
 size_t sdv2_swa_attn_workspace_bytes(int32_t rows, int32_t q_tokens, int32_t heads,

@@ -62,8 +62,9 @@ typedef enum sdv2_stream_mode {
   SDV2_STREAM_LDS_32_ROWS = 1,    /* + LDS fragment reads as the attention kernel makes them:
                                      8 waves x 32 query rows, 1.5 reads per MFMA               */
   SDV2_STREAM_LDS_64_ROWS = 2,    /* the same with 4 waves x 64 query rows: 0.75 reads per MFMA */
-  SDV2_STREAM_ATTENTION_MIX = 3   /* mode 1 + the softmax instructions between the MFMAs + the
+  SDV2_STREAM_ATTENTION_MIX = 3,  /* mode 1 + the softmax instructions between the MFMAs + the
                                      global->LDS tile transfers and the barrier per tile       */
+  SDV2_STREAM_ATTENTION_MIX_64_ROWS = 4   /* mode 2 + the same additions                        */
 } sdv2_stream_mode;
 size_t sdv2_profile_mfma_stream_bytes(void);
 int sdv2_profile_mfma_stream(int mode, const void* operands, size_t operand_bytes, int32_t iterations,

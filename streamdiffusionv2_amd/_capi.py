@@ -12,7 +12,7 @@ from typing import Optional
 
 LIB_PATH = Path(__file__).resolve().parent / "_lib" / "libsdv2kv.so"
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 HEAD_DIM = 128
 MAX_ROWS = 16
 
@@ -29,7 +29,7 @@ DTYPE_BF16 = 0
 DTYPE_F32 = 1
 
 KERNEL_APPEND, KERNEL_ATTENTION, KERNEL_RELAYOUT, KERNEL_SINK, KERNEL_COPY = range(5)
-STREAM_REGISTERS, STREAM_LDS_32_ROWS, STREAM_LDS_64_ROWS, STREAM_ATTENTION_MIX = range(4)
+STREAM_REGISTERS, STREAM_LDS_32_ROWS, STREAM_LDS_64_ROWS, STREAM_ATTENTION_MIX, STREAM_ATTENTION_MIX_64_ROWS = range(5)
 
 # every symbol include/sdv2kv.h and include/sdv2kv_profile.h declare
 EXPORTED_SYMBOLS = (
@@ -81,6 +81,7 @@ class AppendParams(C.Structure):
         ("k_norm_weight", C.c_void_p),
         ("norm_eps", C.c_float),
         ("dst_start_override", C.c_void_p),
+        ("q_inv_rms", C.c_void_p),
     ]
 
 
@@ -103,6 +104,8 @@ class AttnParams(C.Structure):
         ("rope_grid_h", C.c_int32), ("rope_grid_w", C.c_int32),
         ("rope_start_frame", C.POINTER(C.c_int64)),
         ("dtype", C.c_int32),
+        ("q_norm_weight", C.c_void_p),
+        ("q_inv_rms", C.c_void_p),
     ]
 
 

@@ -11,6 +11,7 @@ two HIP kernels and no device-to-host copy.
 from __future__ import annotations
 
 import copy
+import time
 from typing import List, Optional
 
 import torch
@@ -176,7 +177,16 @@ class RingKVPath:
         a reader that comes before they have arrived waits for the stream."""
         refresh = host.tolist()
         if self._NOT_YET in refresh:
+            # The host runs ahead of the stream (it enqueues a layer call in a fraction of the time the GPU
+            # takes for it), so the kernel that writes these words may not have run yet.  Watching the words
+            # lets the host go on the moment they arrive, with the stream still full of work; waiting for the
+            # whole stream would drain it first.
             RingKVPath.decision_waits += 1
+            deadline = time.monotonic() + 2.0
+            while self._NOT_YET in refresh and time.monotonic() < deadline:
+                time.sleep(0)
+                refresh = host.tolist()
+        if self._NOT_YET in refresh:
             stream.synchronize()
             refresh = host.tolist()
             if self._NOT_YET in refresh:
@@ -222,14 +232,19 @@ class RingKVPath:
             for frame in range(dst // frame_tokens, min(self.sink_size, (dst + tokens - 1) // frame_tokens + 1)):
                 kept["stale"][i] |= 1 << frame
 
-    def _layer_launcher(self, q, k, v, kv_cache, table, grid, qk_norm=None):
+    def _layer_launcher(self, q, k, v, kv_cache, table, grid, qk_norm=None, keep_roped_q=False):
         """The cached launch descriptors for this layer, rebuilt when the
-        cache, the shapes, the grid or the norm weights change."""
+        cache, the shapes, the grid or the norm weights change.  keep_roped_q:
+        the caller wants the normalised, rotated query back, so the append
+        writes it (otherwise, with the norm folded in, no such tensor exists)."""
         launcher = getattr(self, "_launcher", None)
+        in_attention = not (keep_roped_q and qk_norm is not None)
         if launcher is None or not launcher.matches(q, k, v, kv_cache, table, qk_norm) \
+                or launcher.rope_in_attention != in_attention \
                 or (launcher.ap.grid_f, launcher.ap.grid_h, launcher.ap.grid_w) != tuple(grid):
             launcher = ops.LayerLauncher(kv_cache["k"], kv_cache["v"], kv_cache["global_end_index"],
-                                         kv_cache["local_end_index"], table, grid, q, k, v, qk_norm=qk_norm)
+                                         kv_cache["local_end_index"], table, grid, q, k, v, qk_norm=qk_norm,
+                                         rope_in_attention=in_attention)
             self._launcher = launcher
         if launcher.forced_splits != self.num_splits:
             launcher.forced_splits = self.num_splits
@@ -330,7 +345,7 @@ class RingKVPath:
             if q.dtype == torch.bfloat16 and rows <= ops._capi.MAX_ROWS:
                 # steady-state fast path: launch descriptors are built once per
                 # (cache, shape) and only patched per call
-                launcher = self._layer_launcher(q, k, v, kv_cache, table, (f, h, w), qk_norm)
+                launcher = self._layer_launcher(q, k, v, kv_cache, table, (f, h, w), qk_norm, return_roped_query)
                 start_frames = [c // frame_tokens for c in starts]
                 out = launcher.launch(q, k, v, start_frames, plan, seq, mask_tokens, override)
                 if return_roped_query:

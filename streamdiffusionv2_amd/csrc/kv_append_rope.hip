@@ -42,6 +42,7 @@ struct AppendKernelArgs {
   int64_t* global_end;
   int64_t* local_end;
   const int64_t* dst_override;              // device [rows] or null; a value >= 0 replaces dst_start[row]
+  float* q_inv_rms;                         // device [rows][tokens] or null: 1 / rms of every q token (fused norm)
   int64_t cache_tokens;
   int32_t tokens, heads, grid_w, frame_tokens;
   int32_t split_t, split_h;                 // pair index bounds: [0,split_t) temporal, [split_t,split_h) height
@@ -128,32 +129,74 @@ void kv_append_rope_kernel(const AppendKernelArgs a) {
 // (WanRMSNorm, wan_base/modules/model.py:70-86, as applied in qkv_fn,
 // causal_model.py:212-218): y = type_as(x.float() * rsqrt(mean(x^2) + eps)) *
 // weight over the full heads * 128 vector of a token, then RoPE and the
-// scatter as above.  One wave per token: lane l owns the 8-element slice
-// l % 16 of heads 4 * j + l / 16 (j = 0, 1, ...) and keeps its q / k slices in
-// registers between the sum of squares and the write.  Rounding steps are the
-// reference's: normalised value to the storage type, times weight to the
-// storage type, rotation in double to float to the storage type.
+// scatter as above.  Rounding steps are the reference's: normalised value to
+// the storage type, times weight to the storage type, rotation in double to
+// float to the storage type.
 //
-// The sum of squares is taken in the order of PyTorch's CPU sum kernel
-// (sdv2::wave_sum_squares), so that mean, rsqrt and everything after them come
-// out bit for bit as on the reference's CPU path.
+// One workgroup of four waves per token.  Heads go in steps of four (lane l
+// of a wave owns the 8-element slice l % 16 of head 4 j + l / 16 of its step
+// j); wave w takes the steps w, w + 4, ... and keeps their q / k slices in
+// registers between the sum of squares and the write.  The sum of squares is
+// taken in the order of PyTorch's CPU sum kernel (ATen cascade_sum /
+// vectorized_inner_sum with 8-float vectors, which the AVX2 and AVX512 builds
+// share), so that mean, rsqrt and everything after them come out bit for bit
+// as on the reference's CPU path: element e of the row belongs to accumulator
+// (e / 8 % 4, e % 8); an accumulator adds its elements in blocks of 16, each
+// block summed in order from zero, the block sums added up in order; a
+// trailing partial block goes first; then the four accumulators of a vector
+// lane are added in order, then the eight lanes in order, starting from zero.
+// With e = 128 head + 8 slice + t the 16 lanes l % 4 == c of a step hold
+// exactly one block of accumulator (c, t), in lane order: every wave parks its
+// step's squares in LDS, lanes 0-31 (k) / 32-63 (q) each walk one accumulator's
+// block, and the block sums meet in LDS, where every wave adds them up in
+// step order.  The caller has checked this order against torch on the CPU.
+//
+// The query is needed for its sum of squares only when q_inv_rms is given:
+// the attention kernel then normalises and rotates the raw query itself
+// (sdv2_attn_params.q_norm_weight / q_inv_rms) and no rotated copy is written.
 // ---------------------------------------------------------------------------
 constexpr int kNormMaxSteps = 16;           // heads <= 64
+constexpr int kNormWaves = 4;
 
-template <typename T, int kSteps>
-__global__ __launch_bounds__(256)
+template <typename T, int kStepsPerWave, bool kWriteQ>
+__global__ __launch_bounds__(64 * kNormWaves)
 void kv_append_norm_rope_kernel(const AppendKernelArgs a) {
+#pragma clang fp contract(off)
   const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
   const int sub = lane & (kLanesPerRow - 1);            // 8-element slice of a head row
   const int head_in_step = lane >> 4;                   // 0..3
-  const int tok = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int tok = blockIdx.x;
   const int row = blockIdx.z;
 
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     if (a.global_end) a.global_end[row] = a.new_global[row];
     if (a.local_end) a.local_end[row] = a.new_local[row];
   }
-  if (tok >= a.tokens) return;                          // whole waves leave together
+
+  const int64_t e0 = sub * 8;
+  const int64_t dst_tok = row_dst_start(a, row) + tok;
+  const T* qi = static_cast<const T*>(a.q_in) + row * a.q_in_st.row + tok * a.q_in_st.token + e0;
+  const T* ki = static_cast<const T*>(a.k_in) + row * a.k_in_st.row + tok * a.k_in_st.token + e0;
+  const T* vi = static_cast<const T*>(a.v_in) + row * a.v_in_st.row + tok * a.v_in_st.token + e0;
+  T* kc = static_cast<T*>(a.k_cache) + row * a.k_st.row + dst_tok * a.k_st.token + e0;
+  T* vc = static_cast<T*>(a.v_cache) + row * a.v_st.row + dst_tok * a.v_st.token + e0;
+  const int steps = (a.heads + 3) >> 2;
+
+  sdv2::Vec8<T> q[kStepsPerWave], k[kStepsPerWave];
+#pragma unroll
+  for (int i = 0; i < kStepsPerWave; ++i) {
+    const int j = wave + kNormWaves * i;
+    const int h = 4 * j + head_in_step;
+    if (j < steps && h < a.heads) {
+      q[i] = sdv2::Vec8<T>::load(qi + h * a.q_in_st.head);
+      k[i] = sdv2::Vec8<T>::load(ki + h * a.k_in_st.head);
+      sdv2::Vec8<T>::load(vi + h * a.v_in_st.head).store(vc + h * a.v_st.head);
+    } else {
+      q[i] = sdv2::Vec8<T>::zero();
+      k[i] = sdv2::Vec8<T>::zero();
+    }
+  }
 
   const int fi = tok / a.frame_tokens;
   const int rem = tok - fi * a.frame_tokens;
@@ -162,45 +205,71 @@ void kv_append_norm_rope_kernel(const AppendKernelArgs a) {
   double2 cs[4];
   sdv2::load_rotation(a.freqs, a.pairs, a.split_t, a.split_h, sub, a.start_frame[row] + fi, hi, wi, cs);
 
-  const int64_t e0 = sub * 8;
-  const int64_t dst_tok = row_dst_start(a, row) + tok;
-  const T* qi = static_cast<const T*>(a.q_in) + row * a.q_in_st.row + tok * a.q_in_st.token + e0;
-  const T* ki = static_cast<const T*>(a.k_in) + row * a.k_in_st.row + tok * a.k_in_st.token + e0;
-  const T* vi = static_cast<const T*>(a.v_in) + row * a.v_in_st.row + tok * a.v_in_st.token + e0;
-  T* qo = static_cast<T*>(a.q_out) + row * a.q_out_st.row + tok * a.q_out_st.token + e0;
-  T* kc = static_cast<T*>(a.k_cache) + row * a.k_st.row + dst_tok * a.k_st.token + e0;
-  T* vc = static_cast<T*>(a.v_cache) + row * a.v_st.row + dst_tok * a.v_st.token + e0;
-  const int steps = (a.heads + 3) >> 2;
-
-  sdv2::Vec8<T> q[kSteps], k[kSteps];
+  __shared__ float squares[kNormWaves][2][64 * 8];     // per wave: one step's squares of k and of q
+  __shared__ float block_sums[2][kNormMaxSteps][32];   // k / q, step, accumulator
+  const int which = lane >> 5;               // lanes 0-31 add up k, lanes 32-63 q
+  const int chain = lane & 31;               // accumulator (c, t) = (chain % 4, chain / 4)
+  const int c = chain & 3, t = chain >> 2;
+  const int full = a.heads >> 2;             // steps whose four heads all exist: whole blocks of 16
+  const int tail = 4 * (a.heads & 3);        // elements of the trailing partial block
 #pragma unroll
-  for (int j = 0; j < kSteps; ++j) {
-    const int h = 4 * j + head_in_step;
-    if (j < steps && h < a.heads) {
-      q[j] = sdv2::Vec8<T>::load(qi + h * a.q_in_st.head);
-      k[j] = sdv2::Vec8<T>::load(ki + h * a.k_in_st.head);
-      sdv2::Vec8<T>::load(vi + h * a.v_in_st.head).store(vc + h * a.v_st.head);
-    } else {
-      q[j] = sdv2::Vec8<T>::zero();
-      k[j] = sdv2::Vec8<T>::zero();
+  for (int i = 0; i < kStepsPerWave; ++i) {
+    const int j = wave + kNormWaves * i;
+    if (j < steps) {                         // (wave-uniform)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        squares[wave][0][lane * 8 + e] = k[i].getf(e) * k[i].getf(e);
+        squares[wave][1][lane * 8 + e] = q[i].getf(e) * q[i].getf(e);
+      }
+      // (LDS operations of one wave complete in order: no barrier between the stores and the loads)
+      const int count = j < full ? 16 : tail;
+      float block = 0.f;
+#pragma unroll
+      for (int m = 0; m < 16; ++m)
+        if (m < count) block += squares[wave][which][(c + 4 * m) * 8 + t];
+      block_sums[which][j][chain] = block;
     }
   }
-  __shared__ float squares[4][2][64 * 8];          // per wave: one step's squares of k and of q
-  float ssq_k, ssq_q;
-  sdv2::wave_sum_squares<T, kSteps>(k, q, a.heads, squares[threadIdx.x >> 6], lane, ssq_k, ssq_q);
+  __syncthreads();
+  float blocks = 0.f;                        // the whole blocks' sums, added up in order
+  for (int j = 0; j < full; ++j) blocks += block_sums[which][j][chain];
+  const float mine = tail ? block_sums[which][full][chain] + blocks : blocks;
+  // the four accumulators of vector lane t, in order: they sit in the four lanes of a quad, whose values
+  // every lane of the quad can take without a trip through LDS
+  auto quad_lane = [](float x, auto which_c) {
+    constexpr int i = decltype(which_c)::value;
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), i | (i << 2) | (i << 4) | (i << 6), 0xf, 0xf, false));
+  };
+  float lane_sum = quad_lane(mine, std::integral_constant<int, 0>{});
+  lane_sum += quad_lane(mine, std::integral_constant<int, 1>{});
+  lane_sum += quad_lane(mine, std::integral_constant<int, 2>{});
+  lane_sum += quad_lane(mine, std::integral_constant<int, 3>{});
+  // the eight vector lanes, in order, from zero: k's in lanes 0, 4, ... 28, q's 32 lanes further up
+  float ssq_k = 0.f, ssq_q = 0.f;
+#pragma unroll
+  for (int v = 0; v < 8; ++v) {
+    ssq_k += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(lane_sum), 4 * v));
+    ssq_q += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(lane_sum), 32 + 4 * v));
+  }
+
   const float width = static_cast<float>(a.heads * 128);
   const float rq = 1.0f / sqrtf(ssq_q / width + a.norm_eps);
   const float rk = 1.0f / sqrtf(ssq_k / width + a.norm_eps);
+  if (a.q_inv_rms && threadIdx.x == 0) a.q_inv_rms[(int64_t)row * a.tokens + tok] = rq;
   const T* wq = static_cast<const T*>(a.q_norm_w) + e0;
   const T* wk = static_cast<const T*>(a.k_norm_w) + e0;
 #pragma unroll
-  for (int j = 0; j < kSteps; ++j) {
+  for (int i = 0; i < kStepsPerWave; ++i) {
+    const int j = wave + kNormWaves * i;
     const int h = 4 * j + head_in_step;
     if (j < steps && h < a.heads) {
-      const sdv2::Vec8<T> qn = sdv2::normalise(q[j], rq, sdv2::Vec8<T>::load(wq + h * 128));
-      const sdv2::Vec8<T> kn = sdv2::normalise(k[j], rk, sdv2::Vec8<T>::load(wk + h * 128));
-      sdv2::rotate(qn, cs).store(qo + h * a.q_out_st.head);
+      const sdv2::Vec8<T> kn = sdv2::normalise(k[i], rk, sdv2::Vec8<T>::load(wk + h * 128));
       sdv2::rotate(kn, cs).store(kc + h * a.k_st.head);
+      if constexpr (kWriteQ) {
+        T* qo = static_cast<T*>(a.q_out) + row * a.q_out_st.row + tok * a.q_out_st.token + e0;
+        const sdv2::Vec8<T> qn = sdv2::normalise(q[i], rq, sdv2::Vec8<T>::load(wq + h * 128));
+        sdv2::rotate(qn, cs).store(qo + h * a.q_out_st.head);
+      }
     }
   }
 }
@@ -223,7 +292,11 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
   if (p->grid_f <= 0 || p->grid_h <= 0 || p->grid_w <= 0) return SDV2_ERR_INVALID_ARG;
   if (static_cast<int64_t>(p->grid_f) * p->grid_h * p->grid_w != p->tokens) return SDV2_ERR_INVALID_ARG;
   if (!p->freqs) return SDV2_ERR_INVALID_ARG;
-  if ((p->q_in == nullptr) != (p->q_out == nullptr)) return SDV2_ERR_INVALID_ARG;
+  const bool with_norm = p->q_norm_weight != nullptr || p->k_norm_weight != nullptr;
+  // q comes with the tensor its rotation goes to - or, with the norm folded in, with the place for its 1 / rms
+  if (p->q_inv_rms && !with_norm) return SDV2_ERR_INVALID_ARG;
+  if (p->q_in == nullptr ? (p->q_out != nullptr || p->q_inv_rms != nullptr) : (p->q_out == nullptr && p->q_inv_rms == nullptr))
+    return SDV2_ERR_INVALID_ARG;
   const bool with_q = p->q_in != nullptr;
   // k, v and the two caches come together or not at all; without them the call
   // only rotates q (and then has nothing to do with a cache or its indices)
@@ -236,13 +309,13 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
   if (!p->start_frame || (with_kv && !p->dst_start)) return SDV2_ERR_INVALID_ARG;
   if ((p->global_end_index || p->local_end_index) && (!p->new_global_end || !p->new_local_end))
     return SDV2_ERR_INVALID_ARG;
-  const bool with_norm = p->q_norm_weight != nullptr || p->k_norm_weight != nullptr;
   if (with_norm) {
     // the fused norm covers q and k together, as qkv_fn applies it
     if (!p->q_norm_weight || !p->k_norm_weight || !with_q) return SDV2_ERR_INVALID_ARG;
     if (p->heads > 4 * kNormMaxSteps) return SDV2_ERR_UNSUPPORTED;
     if (!(p->norm_eps >= 0.f)) return SDV2_ERR_INVALID_ARG;
     if (!aligned16(p->q_norm_weight) || !aligned16(p->k_norm_weight)) return SDV2_ERR_INVALID_ARG;
+    if (p->q_inv_rms && (reinterpret_cast<uintptr_t>(p->q_inv_rms) & 3)) return SDV2_ERR_INVALID_ARG;
   }
 
   // 16-byte vector access: 8 bf16 or 4 floats per transaction.
@@ -253,7 +326,7 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
   if (with_kv && (!stride_ok(p->k_in_stride, vec) || !stride_ok(p->v_in_stride, vec) ||
                   !stride_ok(p->k_cache_stride, vec) || !stride_ok(p->v_cache_stride, vec)))
     return SDV2_ERR_INVALID_ARG;
-  if (with_q && (!stride_ok(p->q_in_stride, vec) || !stride_ok(p->q_out_stride, vec)))
+  if (with_q && (!stride_ok(p->q_in_stride, vec) || (p->q_out && !stride_ok(p->q_out_stride, vec))))
     return SDV2_ERR_INVALID_ARG;
 
   if (p->grid_h > p->freq_rows || p->grid_w > p->freq_rows) return SDV2_ERR_OUT_OF_RANGE;
@@ -273,6 +346,7 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
   a.global_end = p->global_end_index;
   a.local_end = p->local_end_index;
   a.dst_override = p->dst_start_override;
+  a.q_inv_rms = p->q_inv_rms;
   a.cache_tokens = p->cache_tokens;
   a.tokens = p->tokens; a.heads = p->heads; a.grid_w = p->grid_w;
   a.frame_tokens = p->grid_h * p->grid_w;
@@ -293,19 +367,24 @@ extern "C" int sdv2_kv_append_rope(const sdv2_append_params* p) {
             (p->heads + kHeadsPerThread - 1) / kHeadsPerThread, p->rows);
   hipStream_t stream = static_cast<hipStream_t>(p->stream);
   if (with_norm) {
-    const dim3 norm_grid((p->tokens + 3) / 4, 1, p->rows);
-    // the q / k slices of a token stay in registers: the variant fixes how many heads / 4 fit
+    const dim3 norm_grid(p->tokens, 1, p->rows);
+    const dim3 norm_block(64 * kNormWaves);
+    // the q / k slices of a wave's steps stay in registers: the variant fixes how many steps a wave takes
     auto launch = [&](auto steps_c) {
       constexpr int kS = decltype(steps_c)::value;
-      if (p->dtype == SDV2_BF16)
-        sdv2::launch_timed(SDV2_KERNEL_APPEND, kv_append_norm_rope_kernel<uint16_t, kS>, norm_grid, block, 0, stream, a);
-      else
-        sdv2::launch_timed(SDV2_KERNEL_APPEND, kv_append_norm_rope_kernel<float, kS>, norm_grid, block, 0, stream, a);
+      const bool write_q = p->q_out != nullptr;
+      if (p->dtype == SDV2_BF16) {
+        if (write_q) sdv2::launch_timed(SDV2_KERNEL_APPEND, kv_append_norm_rope_kernel<uint16_t, kS, true>, norm_grid, norm_block, 0, stream, a);
+        else sdv2::launch_timed(SDV2_KERNEL_APPEND, kv_append_norm_rope_kernel<uint16_t, kS, false>, norm_grid, norm_block, 0, stream, a);
+      } else {
+        if (write_q) sdv2::launch_timed(SDV2_KERNEL_APPEND, kv_append_norm_rope_kernel<float, kS, true>, norm_grid, norm_block, 0, stream, a);
+        else sdv2::launch_timed(SDV2_KERNEL_APPEND, kv_append_norm_rope_kernel<float, kS, false>, norm_grid, norm_block, 0, stream, a);
+      }
     };
-    const int steps = (p->heads + 3) / 4;
-    if (steps <= 4) launch(std::integral_constant<int, 4>{});
-    else if (steps <= 10) launch(std::integral_constant<int, 10>{});
-    else launch(std::integral_constant<int, kNormMaxSteps>{});
+    const int per_wave = ((p->heads + 3) / 4 + kNormWaves - 1) / kNormWaves;
+    if (per_wave <= 1) launch(std::integral_constant<int, 1>{});
+    else if (per_wave <= 3) launch(std::integral_constant<int, 3>{});
+    else launch(std::integral_constant<int, kNormMaxSteps / kNormWaves>{});
     return hipGetLastError() == hipSuccess ? SDV2_OK : SDV2_ERR_LAUNCH;
   }
   auto launch = [&](auto kernel) {

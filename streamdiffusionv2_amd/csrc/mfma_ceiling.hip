@@ -19,6 +19,9 @@
 //                 between the MFMAs (fma, exp2, pack, row sum; the weights they
 //                 produce are the B operands of the following block) + the
 //                 global->LDS tile transfers and the barrier per 64-key tile
+//   mix, 64 rows  the same additions on the 64-rows-per-wave stream: what a
+//                 re-blocking of the attention kernel to two query blocks per
+//                 wave could reach in its loop
 //
 // The distance between "attention mix" and the attention kernel's own rate is
 // what the kernel loses outside its loop (prologue, partial results, combine,
@@ -357,12 +360,17 @@ void mfma_stream32_kernel(const StreamArgs a) {
 }
 
 // 4 waves x 64 query rows (one wave per SIMD, 512 registers): two query blocks
-// per wave, every K and V^T fragment feeds one MFMA of each.
+// per wave, every K and V^T fragment feeds one MFMA of each.  kSoftmax / kDma
+// add what they add to the 32-row kernel: the softmax instructions of both
+// blocks between the MFMAs, the tile transfers (all four waves issue) and the
+// barrier per tile.
+template <bool kSoftmax, bool kDma>
 __global__ __launch_bounds__(256, 1)
 void mfma_stream64_kernel(const StreamArgs a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   lds_char* lds = (lds_char*)smem;
   const int tid = threadIdx.x, lane = tid & 63;
+  const int wave_u = __builtin_amdgcn_readfirstlane(tid >> 6);
   fill_lds<256>(lds, a.operands, tid);
   const LaneAddr c = lane_addresses(lane);
   bf16x8 qf[2][8];
@@ -391,6 +399,27 @@ void mfma_stream64_kernel(const StreamArgs a) {
 #pragma unroll
     for (int i = 0; i < 16; ++i) { s[b][0][i] = 0.f; s[b][1][i] = 0.f; }
   }
+  float l[2] = {0.f, 0.f};
+  float c2 = 1.4427f, neg_ref = -4.0f;
+  pin(c2);
+  pin(neg_ref);
+
+  const char* region = a.operands + kStreamOff + (size_t)(blockIdx.x % kRegions) * kRegionBytes;
+  {
+    const uint64_t x = reinterpret_cast<uint64_t>(region);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)x), hi = __builtin_amdgcn_readfirstlane((uint32_t)(x >> 32));
+    region = reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
+  }
+  uint32_t ld[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) ld[j] = (uint32_t)((wave_u * 4 + j) * 1024 + lane * 16);
+  auto issue = [&](int T, int buf, int is_v) {
+    const char* tile = region + (size_t)(T % kRegionTiles) * (2 * kTileBytes) + is_v * kTileBytes;
+    const uint32_t dst = (uint32_t)((is_v ? 3 : 0) * kTileBytes + buf * kTileBytes);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) dma16(tile, ld[j], dst + (wave_u * 4 + j) * 1024);
+  };
+
   auto slot = [&](auto par_c, auto koff_c, auto voff_c) {
     constexpr int kPar = decltype(par_c)::value, kKOff = decltype(koff_c)::value, kVOff = decltype(voff_c)::value;
     u32x4 kfrag[8], vfrag[8];
@@ -401,37 +430,84 @@ void mfma_stream64_kernel(const StreamArgs a) {
       vfrag[g] = lds_read_tr16_b64x2<kVOff + kk * 16 * 256 - 3 * kTileBytes, g % 3, 240>(c.v[db][0], c.v[db][1]);
     };
     request(std::integral_constant<int, 0>{});
-    static_for<8>([&](auto gc) {
-      constexpr int g = decltype(gc)::value;
-      constexpr int later = (g + 1 < 8 ? 1 : 0) * 3;
-      if constexpr (g + 1 < 8) request(std::integral_constant<int, g + 1>{});
-      if constexpr (g == 0) {
-        mfma_s_first<later + 2>(s[0][kPar], kfrag[g], qf[0][g]);
-        mfma_s_first<later + 2>(s[1][kPar], kfrag[g], qf[1][g]);
-      } else {
-        mfma_s<later + 2>(s[0][kPar], kfrag[g], qf[0][g]);
-        mfma_s<later + 2>(s[1][kPar], kfrag[g], qf[1][g]);
+    __builtin_amdgcn_sched_barrier(0);
+    // 32 steps, one MFMA each: group g = t / 4 runs S of block 0, S of block 1, PV of block 0, PV of block 1;
+    // score u = t (block u / 16, accumulator register u % 16) goes through fma -> exp2 -> pack + row sum one step apart
+    float scaled[33], weight[33];
+    auto softmax_step = [&](auto tc) {
+      constexpr int t = decltype(tc)::value;
+      if constexpr (kSoftmax) {
+        if constexpr (t < 32) {
+          scaled[t] = __builtin_fmaf(s[t >> 4][kPar][t & 15], c2, neg_ref);
+          pin(scaled[t]);
+        }
+        if constexpr (t >= 1 && t - 1 < 32) {
+          weight[t - 1] = __builtin_amdgcn_exp2f(scaled[t - 1]);
+          pin(weight[t - 1]);
+        }
+        if constexpr (t >= 2 && t - 2 < 32 && ((t - 2) & 1) == 1) {
+          constexpr int u = t - 2, b = u >> 4, g = (u & 15) / 2;
+          uint32_t packed = pack_bf16x2(weight[u - 1], weight[u]);
+          l[b] = add_bf16_pair(packed, l[b]);
+          pin(packed);
+          pin(l[b]);
+          p[b][kPar][g >> 2][g & 3] = packed;
+        }
       }
-      mfma_o<later>(oacc[0][g & 3], vfrag[g], p[0][kPar][g >> 2]);
-      mfma_o<later>(oacc[1][g & 3], vfrag[g], p[1][kPar][g >> 2]);
+    };
+    static_for<32>([&](auto tc) {
+      constexpr int t = decltype(tc)::value;
+      constexpr int g = t / 4, i = t % 4;
+      constexpr int later = (g + 1 < 8 ? 1 : 0) * 3;
+      if constexpr (i == 0 && g + 1 < 8) request(std::integral_constant<int, g + 1>{});
+      if constexpr (i < 2) {
+        if constexpr (g == 0) mfma_s_first<later + 2>(s[i][kPar ^ 1], kfrag[g], qf[i][g]);
+        else mfma_s<later + 2>(s[i][kPar ^ 1], kfrag[g], qf[i][g]);
+      } else {
+        mfma_o<later>(oacc[i - 2][g & 3], vfrag[g], p[i - 2][kPar ^ 1][g >> 2]);
+      }
+      softmax_step(tc);
       __builtin_amdgcn_sched_barrier(0);
     });
+    softmax_step(std::integral_constant<int, 32>{});
+    softmax_step(std::integral_constant<int, 33>{});
   };
   using I0 = std::integral_constant<int, 0>;
   using I1 = std::integral_constant<int, 1>;
-  for (int it = 0; it < a.iterations; ++it) {
-    slot(I0{}, std::integral_constant<int, 0>{}, std::integral_constant<int, 3 * kTileBytes + 8192>{});
-    slot(I1{}, std::integral_constant<int, 8192>{}, std::integral_constant<int, 3 * kTileBytes>{});
-    slot(I0{}, std::integral_constant<int, kTileBytes>{}, std::integral_constant<int, 4 * kTileBytes + 8192>{});
-    slot(I1{}, std::integral_constant<int, kTileBytes + 8192>{}, std::integral_constant<int, 4 * kTileBytes>{});
-    slot(I0{}, std::integral_constant<int, 2 * kTileBytes>{}, std::integral_constant<int, 5 * kTileBytes + 8192>{});
-    slot(I1{}, std::integral_constant<int, 2 * kTileBytes + 8192>{}, std::integral_constant<int, 5 * kTileBytes>{});
+  using I2 = std::integral_constant<int, 2>;
+  auto do_tile = [&](auto buf_c, int T) {
+    constexpr int kB = decltype(buf_c)::value;
+    constexpr int kBNext = (kB + 1) % 3, kBPrev = (kB + 2) % 3;
+    slot(I0{}, std::integral_constant<int, kB * kTileBytes + 8192>{},
+         std::integral_constant<int, (3 + kBPrev) * kTileBytes + 8192>{});
+    if constexpr (kDma) {
+      __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
+      __syncthreads();
+      issue(T + 3, kB, 0);
+      issue(T + 2, kBPrev, 1);
+    }
+    slot(I1{}, std::integral_constant<int, kBNext * kTileBytes>{}, std::integral_constant<int, (3 + kB) * kTileBytes>{});
+  };
+  if constexpr (kDma) {
+    issue(0, 0, 0);
+    issue(0, 0, 1);
+    issue(1, 1, 0);
+    issue(1, 1, 1);
+    issue(2, 2, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70 | 8);
+    __syncthreads();
   }
+  for (int it = 0; it < a.iterations; ++it) {
+    do_tile(I0{}, 3 * it);
+    do_tile(I1{}, 3 * it + 1);
+    do_tile(I2{}, 3 * it + 2);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);
   asm volatile("s_nop 15\n\ts_nop 15"
                : "+a"(oacc[0][0]), "+a"(oacc[0][1]), "+a"(oacc[0][2]), "+a"(oacc[0][3]), "+a"(oacc[1][0]), "+a"(oacc[1][1]),
                  "+a"(oacc[1][2]), "+a"(oacc[1][3]));
   asm volatile("" : "+v"(s[0][0]), "+v"(s[0][1]), "+v"(s[1][0]), "+v"(s[1][1]));
-  float acc = 0.f;
+  float acc = l[0] + l[1];
 #pragma unroll
   for (int b = 0; b < 2; ++b)
 #pragma unroll
@@ -461,7 +537,7 @@ extern "C" int sdv2_profile_mfma_stream(int mode, const void* operands, size_t o
   if (reinterpret_cast<uintptr_t>(operands) & 255) return SDV2_ERR_INVALID_ARG;
   int device = 0;
   if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return SDV2_ERR_LAUNCH;
-  static std::atomic<bool> ready[4][kMaxDevices];
+  static std::atomic<bool> ready[5][kMaxDevices];
   StreamArgs a;
   a.operands = static_cast<const char*>(operands);
   a.sink = reinterpret_cast<float*>(const_cast<char*>(a.operands) + kOperandBytes);
@@ -482,8 +558,13 @@ extern "C" int sdv2_profile_mfma_stream(int mode, const void* operands, size_t o
       mfma_per_launch = (double)kCus * 8 * 96 * iterations;
       break;
     case SDV2_STREAM_LDS_64_ROWS:
-      if (!allow_lds(mfma_stream64_kernel, ready[2][device])) return SDV2_ERR_LAUNCH;
-      hipLaunchKernelGGL(mfma_stream64_kernel, dim3(kCus), dim3(256), kLdsBytes, s, a);
+      if (!allow_lds(mfma_stream64_kernel<false, false>, ready[2][device])) return SDV2_ERR_LAUNCH;
+      hipLaunchKernelGGL((mfma_stream64_kernel<false, false>), dim3(kCus), dim3(256), kLdsBytes, s, a);
+      mfma_per_launch = (double)kCus * 4 * 192 * iterations;
+      break;
+    case SDV2_STREAM_ATTENTION_MIX_64_ROWS:
+      if (!allow_lds(mfma_stream64_kernel<true, true>, ready[4][device])) return SDV2_ERR_LAUNCH;
+      hipLaunchKernelGGL((mfma_stream64_kernel<true, true>), dim3(kCus), dim3(256), kLdsBytes, s, a);
       mfma_per_launch = (double)kCus * 4 * 192 * iterations;
       break;
     case SDV2_STREAM_ATTENTION_MIX:

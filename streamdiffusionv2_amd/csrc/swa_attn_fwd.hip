@@ -116,7 +116,11 @@ struct AttnKernelArgs {
   uint16_t* out;
   const int32_t* seq_lens;
   sdv2_stride3 q_st, k_st, v_st, o_st;
-  int32_t rows, q_tokens, heads, max_seq_len, num_splits;
+  int32_t rows, q_tokens, heads, max_seq_len;
+  // Key ranges per (row, head): num_splits, except that of every group_pairs
+  // consecutive (row, head) pairs the last more_pairs take num_splits + 1.
+  // (Uniform: group_pairs = rows * heads, more_pairs = 0.)
+  int32_t num_splits, group_pairs, more_pairs;
   float scale_log2;            // softmax_scale * log2(e)
   int32_t mask_block_tokens;   // 0 = no mask inside the chunk
   const int32_t* chunk_start;  // device [rows]: cache position of the chunk's own first key
@@ -132,6 +136,10 @@ struct AttnKernelArgs {
   const double2* freqs;
   int32_t grid_w, frame_tokens, split_t, split_h;
   int64_t start_frame[SDV2_MAX_ROWS];
+  // RMSNorm of the queries inside the kernel (q is then the raw projection):
+  // the norm weight [heads * 128] and 1 / rms per (row, token), or null
+  const uint16_t* q_norm_w;
+  const float* q_inv_rms;
 };
 
 __device__ __forceinline__ int swz(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
@@ -602,6 +610,12 @@ struct QueryRope {
   const double2* freqs;        // null: the query arrives rotated
   int64_t start_frame;         // of this cache row
   int32_t grid_w, frame_tokens, split_t, split_h;
+  // With norm_w (this head's 128 norm weights, offset like qp) the row is the
+  // raw q projection: every slice is normalised with the token's 1 / rms as
+  // the append kernel's fused norm would have done it (sdv2::normalise: two
+  // roundings to bf16), then rotated.
+  const uint16_t* norm_w;
+  float inv_rms;
 };
 
 __device__ __forceinline__ void load_query(const QueryRope& rope, const uint16_t* qp, int token, int hf,
@@ -619,7 +633,9 @@ __device__ __forceinline__ void load_query(const QueryRope& rope, const uint16_t
     for (int ks = 0; ks < 8; ++ks) {
       double2 cs[4];
       sdv2::load_rotation(rope.freqs, kD / 2, rope.split_t, rope.split_h, 2 * ks + hf, frame, hi, wi, cs);
-      const sdv2::Vec8<uint16_t> y = sdv2::rotate(sdv2::Vec8<uint16_t>::load(qp + 16 * ks), cs);
+      sdv2::Vec8<uint16_t> x = sdv2::Vec8<uint16_t>::load(qp + 16 * ks);
+      if (rope.norm_w) x = sdv2::normalise(x, rope.inv_rms, sdv2::Vec8<uint16_t>::load(rope.norm_w + 16 * ks));
+      const sdv2::Vec8<uint16_t> y = sdv2::rotate(x, cs);
       qf[ks] = __builtin_bit_cast(bf16x8, y.raw);
     }
   }
@@ -644,28 +660,47 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   // head, key split) are neighbours, and XCD x takes the x-th eighth of that
   // list: the workgroups that stream the same K / V run on the same XCD at the
   // same time and all but the first fetch of a tile hit in L2.
-  int qtile, head, row, split;
+  //
+  // With a mixed split count a group of (row, head) pairs is one XCD's share:
+  // its pairs with fewer, longer key ranges come first, so that the workgroups
+  // the dispatcher hands out last are the short ones (longest first is what
+  // packs unequal pieces best onto the CUs).
+  int qtile, head, row, split, nsplits;
   const int nq = (a.q_tokens + kQTile - 1) / kQTile;
   {
-    const int total = nq * a.heads * a.rows * a.num_splits;
+    const int per_lo = nq * a.num_splits, per_hi = per_lo + nq;
+    const int lo_pairs = a.group_pairs - a.more_pairs;
+    const int per_group = lo_pairs * per_lo + a.more_pairs * per_hi;
+    const int total = (a.heads * a.rows / a.group_pairs) * per_group;
     const int xcd = blockIdx.x & 7;
     const int first = (int)(((int64_t)xcd * total) >> 3);
     const int end = (int)(((int64_t)(xcd + 1) * total) >> 3);
-    int item = first + (blockIdx.x >> 3);
+    const int item = first + (blockIdx.x >> 3);
     if (item >= end) return;
-    qtile = item % nq;
-    item /= nq;
-    split = item % a.num_splits;
-    item /= a.num_splits;
-    head = item % a.heads;
-    row = item / a.heads;
+    const int group = item / per_group;
+    int r = item - group * per_group;
+    int pair = group * a.group_pairs;
+    if (r < lo_pairs * per_lo) {
+      nsplits = a.num_splits;
+      pair += r / per_lo;
+      r %= per_lo;
+    } else {
+      nsplits = a.num_splits + 1;
+      r -= lo_pairs * per_lo;
+      pair += lo_pairs + r / per_hi;
+      r %= per_hi;
+    }
+    qtile = r % nq;
+    split = r / nq;
+    head = pair % a.heads;
+    row = pair / a.heads;
   }
 
   int seq = a.seq_lens ? a.seq_lens[row] : a.max_seq_len;
   seq = seq < a.max_seq_len ? seq : a.max_seq_len;
   seq = seq < 0 ? 0 : seq;
   const int ntiles = (seq + kKTile - 1) / kKTile;
-  const int per_split = (ntiles + a.num_splits - 1) / a.num_splits;
+  const int per_split = (ntiles + nsplits - 1) / nsplits;
   const int tile_begin = split * per_split;
   int tile_end = tile_begin + per_split;
   tile_end = tile_end < ntiles ? tile_end : ntiles;
@@ -731,6 +766,8 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
       constexpr int i = decltype(ic)::value + 1;
       rope.start_frame = row == i ? a.start_frame[i] : rope.start_frame;
     });
+    rope.norm_w = a.q_norm_w ? a.q_norm_w + head * kD + 8 * hf : nullptr;
+    rope.inv_rms = a.q_norm_w ? a.q_inv_rms[(int64_t)row * a.q_tokens + q_row_c] : 1.0f;
     load_query(rope, a.q + row * a.q_st.row + (int64_t)q_row_c * a.q_st.token + head * a.q_st.head + 8 * hf, q_row_c,
                hf, qf);
   }
@@ -925,7 +962,7 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   float l_tot = half_sum(l_run);
   float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
 
-  if (a.num_splits > 1) {
+  if (nsplits > 1) {
     // Partial result of a key range: the normalised row divided by its largest
     // magnitude, as fp16 (values in [-1, 1]: 11 bits against the row's scale,
     // sixteen times finer than the bf16 of the final result), plus that scale
@@ -974,7 +1011,7 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
     if (tid == 0) {
       int32_t* ticket = a.tickets + ((int64_t)row * a.heads + head) * nq + qtile;
       const int drawn = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const int last = drawn == a.num_splits - 1;
+      const int last = drawn == nsplits - 1;
       if (last) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       *reinterpret_cast<lds_int*>(lds) = last;
     }
@@ -993,7 +1030,7 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
     auto fetch = [&](int s0) {
 #pragma unroll
       for (int u = 0; u < kBatch; ++u) {
-        const int sp = s0 + u < a.num_splits ? s0 + u : a.num_splits - 1;
+        const int sp = s0 + u < nsplits ? s0 + u : nsplits - 1;
         lse[u] = load_coherent(a.part_lse + (sp * slab + blk0) * kQBlock + r32);
         scale[u] = load_coherent(a.part_scale + (sp * slab + blk0) * kQBlock + r32);
       }
@@ -1002,23 +1039,23 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
     float lse_max = lse[0];
 #pragma unroll
     for (int u = 1; u < kBatch; ++u) lse_max = fmaxf(lse_max, lse[u]);         // (entries past the last range repeat it)
-    for (int sp = kBatch; sp < a.num_splits; ++sp)
+    for (int sp = kBatch; sp < nsplits; ++sp)
       lse_max = fmaxf(lse_max, load_coherent(a.part_lse + (sp * slab + blk0) * kQBlock + r32));
 #pragma unroll
     for (int db = 0; db < 4; ++db)
 #pragma unroll
       for (int i = 0; i < 16; ++i) oacc[db][i] = 0.f;
-    for (int s0 = 0; s0 < a.num_splits; s0 += kBatch) {
+    for (int s0 = 0; s0 < nsplits; s0 += kBatch) {
       if (s0 > 0) fetch(s0);
 #pragma unroll
       for (int u = 0; u < kBatch; ++u) {
-        const float w = (s0 + u >= a.num_splits || lse[u] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(lse[u] - lse_max);
+        const float w = (s0 + u >= nsplits || lse[u] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(lse[u] - lse_max);
         wsum += w;
         ws[u] = w * scale[u];         // weight times the row's fp16 scale
       }
 #pragma unroll
       for (int u = 0; u < kBatch; ++u) {
-        if (s0 + u >= a.num_splits) break;
+        if (s0 + u >= nsplits) break;
         u32x4 x[8];
         load_coherent_x8(
             reinterpret_cast<const char*>(a.part_o + ((s0 + u) * slab + blk0) * kPartBlockHalves + lane * 8), x);
@@ -1121,6 +1158,27 @@ void* static_scratch_address() {
 
 int attn_fwd(const sdv2_attn_params* p, void* workspace, size_t workspace_bytes);
 
+// How a call's key ranges are cut, as num_splits carries it: bits 0-7 the
+// count s every (row, head) pair gets at least, bits 8-15 how many of the
+// pairs of each eighth of the (row, head) list (one XCD's share) get s + 1.
+struct SplitPlan {
+  int base, more, group;
+  int most() const { return base + (more > 0 ? 1 : 0); }
+};
+bool decode_splits(int32_t encoded, int32_t rows, int32_t heads, SplitPlan* plan) {
+  if (encoded <= 0 || (encoded >> 16) != 0) return false;
+  plan->base = encoded & 0xff;
+  plan->more = (encoded >> 8) & 0xff;
+  const int64_t pairs = (int64_t)rows * heads;
+  plan->group = (int)pairs;
+  if (plan->base < 1) return false;
+  if (plan->more > 0) {
+    if (pairs % 8 != 0 || plan->more >= pairs / 8) return false;
+    plan->group = (int)(pairs / 8);
+  }
+  return plan->most() <= 64;
+}
+
 }  // namespace
 
 extern "C" int sdv2_swa_attn_default_splits(int32_t rows, int32_t q_tokens, int32_t heads, int32_t max_seq_len) {
@@ -1131,8 +1189,20 @@ extern "C" int sdv2_swa_attn_default_splits(int32_t rows, int32_t q_tokens, int3
   // times.  Writing and combining the partial results
   // costs roughly one tile time per 3.5 MB of them per split.  Constants fitted
   // to measurements on the five benchmark shapes.
-  const int64_t qwork = (int64_t)rows * heads * ((q_tokens + kQTile - 1) / kQTile);
+  const int nq = (q_tokens + kQTile - 1) / kQTile;
+  const int64_t pairs = (int64_t)rows * heads;
+  const int64_t qwork = pairs * nq;
   if (qwork > kMaxTickets) return 1;
+  // (the answer depends on the shape alone and costs a small simulation: the last one is remembered)
+  static std::mutex lock;
+  static int32_t last_shape[4] = {0, 0, 0, 0};
+  static int last_answer = 0;
+  {
+    std::lock_guard<std::mutex> guard(lock);
+    if (last_answer && last_shape[0] == rows && last_shape[1] == q_tokens && last_shape[2] == heads &&
+        last_shape[3] == max_seq_len)
+      return last_answer;
+  }
   const int ntiles = (max_seq_len + kKTile - 1) / kKTile;
   const double partial_tiles = (double)rows * heads * q_tokens * kD * 4 / 7.0e6;
   int best = 1;
@@ -1144,14 +1214,55 @@ extern "C" int sdv2_swa_attn_default_splits(int32_t rows, int32_t q_tokens, int3
     const double cost = (double)rounds * (per + 3) + (sp > 1 ? sp * partial_tiles : 0.0);
     if (cost < best_cost - 1e-9) { best_cost = cost; best = sp; }
   }
+  // A uniform count can leave the last round of workgroups mostly empty (1120
+  // workgroups are 4.4 rounds of 256).  When the (row, head) pairs divide over
+  // the eight XCDs, some pairs of each XCD's share may take one range more:
+  // workgroups of two lengths, the long ones dispatched first, fill the 32 CUs
+  // of an XCD more evenly.  Simulated as the dispatcher works (next workgroup
+  // to the CU that is free first); taken when it beats the best uniform count
+  // by 3 %.
+  if (pairs % 8 == 0 && pairs / 8 >= 2 && pairs / 8 <= 255) {
+    const int group = (int)(pairs / 8);
+    constexpr int kCusPerXcd = kCuSlots / 8;
+    double mixed_cost = 1e300;
+    int mixed = 0;
+    for (int sp = 1; sp <= 7; ++sp) {
+      const int per_lo = (ntiles + sp - 1) / sp, per_hi = (ntiles + sp) / (sp + 1);
+      if (per_hi < 6) break;
+      for (int more = 1; more < group; ++more) {
+        double busy[kCusPerXcd] = {};
+        auto hand_out = [&](int count, double length) {
+          for (int i = 0; i < count; ++i) {
+            int cu = 0;
+            for (int c = 1; c < kCusPerXcd; ++c)
+              if (busy[c] < busy[cu]) cu = c;
+            busy[cu] += length;
+          }
+        };
+        hand_out((group - more) * nq * sp, per_lo + 3);
+        hand_out(more * nq * (sp + 1), per_hi + 3);
+        double span = 0;
+        for (double b : busy) span = b > span ? b : span;
+        const double ranges = ((double)(group - more) * sp + (double)more * (sp + 1)) / group;
+        const double cost = span + ranges * partial_tiles;
+        if (cost < mixed_cost - 1e-9) { mixed_cost = cost; mixed = sp | (more << 8); }
+      }
+    }
+    if (mixed_cost < 0.97 * best_cost) best = mixed;
+  }
+  std::lock_guard<std::mutex> guard(lock);
+  last_shape[0] = rows; last_shape[1] = q_tokens; last_shape[2] = heads; last_shape[3] = max_seq_len;
+  last_answer = best;
   return best;
 }
 
 extern "C" size_t sdv2_swa_attn_workspace_bytes(int32_t rows, int32_t q_tokens, int32_t heads,
                                                  int32_t max_seq_len, int32_t num_splits) {
+  if (rows <= 0 || q_tokens <= 0 || heads <= 0) return 0;
   if (num_splits <= 0) num_splits = sdv2_swa_attn_default_splits(rows, q_tokens, heads, max_seq_len);
-  if (num_splits <= 1 || rows <= 0 || q_tokens <= 0 || heads <= 0) return 0;
-  return workspace_layout(rows, q_tokens, heads, num_splits).total;
+  SplitPlan plan;
+  if (!decode_splits(num_splits, rows, heads, &plan) || plan.most() <= 1) return 0;
+  return workspace_layout(rows, q_tokens, heads, plan.most()).total;
 }
 
 extern "C" int sdv2_swa_attn_fwd(const sdv2_attn_params* p) {
@@ -1164,10 +1275,11 @@ extern "C" int sdv2_swa_attn_fwd_static(const sdv2_attn_params* p) {
   if (p->rows <= 0 || p->q_tokens <= 0 || p->heads <= 0 || p->max_seq_len < 0)
     return attn_fwd(p, nullptr, 0);                       // nothing to split: same answers as the plain entry point
   if (p->dtype == SDV2_F32) return attn_fwd(p, nullptr, 0);   // fp32 walks one key range: no scratch, whatever num_splits says
-  if (p->num_splits > 64) return SDV2_ERR_INVALID_ARG;        // as the plain entry point answers
   const int splits = p->num_splits > 0 ? p->num_splits
                                        : sdv2_swa_attn_default_splits(p->rows, p->q_tokens, p->heads, p->max_seq_len);
-  if (splits <= 1) return attn_fwd(p, nullptr, 0);
+  SplitPlan plan;
+  if (!decode_splits(splits, p->rows, p->heads, &plan)) return SDV2_ERR_INVALID_ARG;   // as the plain entry point answers
+  if (plan.most() <= 1) return attn_fwd(p, nullptr, 0);
   if (sdv2_swa_attn_workspace_bytes(p->rows, p->q_tokens, p->heads, p->max_seq_len, splits) >
       (size_t)SDV2_STATIC_SCRATCH_BYTES)
     return SDV2_ERR_SCRATCH_LIMIT;
@@ -1191,9 +1303,12 @@ int attn_fwd(const sdv2_attn_params* p, void* workspace, size_t workspace_bytes)
     return SDV2_ERR_INVALID_ARG;
   if (p->rows > 65535 / 8 || p->heads > 65535) return SDV2_ERR_INVALID_ARG;
 
-  int splits = p->num_splits > 0 ? p->num_splits
-                                 : sdv2_swa_attn_default_splits(p->rows, p->q_tokens, p->heads, p->max_seq_len);
-  if (splits > 64) return SDV2_ERR_INVALID_ARG;
+  SplitPlan plan;
+  if (!decode_splits(p->num_splits > 0 ? p->num_splits
+                                       : sdv2_swa_attn_default_splits(p->rows, p->q_tokens, p->heads, p->max_seq_len),
+                     p->rows, p->heads, &plan))
+    return SDV2_ERR_INVALID_ARG;
+  const int splits = plan.most();
   if ((int64_t)p->rows * splits > 65535) return SDV2_ERR_INVALID_ARG;
   // more (row, head, query tile) groups than there are ticket words: such a grid fills the chip unsplit
   if (splits > 1 && (int64_t)p->rows * p->heads * ((p->q_tokens + kQTile - 1) / kQTile) > kMaxTickets)
@@ -1207,7 +1322,9 @@ int attn_fwd(const sdv2_attn_params* p, void* workspace, size_t workspace_bytes)
   a.seq_lens = p->seq_lens;
   a.q_st = p->q_stride; a.k_st = p->k_stride; a.v_st = p->v_stride; a.o_st = p->out_stride;
   a.rows = p->rows; a.q_tokens = p->q_tokens; a.heads = p->heads; a.max_seq_len = p->max_seq_len;
-  a.num_splits = splits;
+  a.num_splits = plan.base;
+  a.group_pairs = plan.group;
+  a.more_pairs = plan.more;
   const float scale = p->softmax_scale > 0.f ? p->softmax_scale : 0.08838834764831845f;  // 1/sqrt(128)
   a.scale_log2 = scale * kLog2e;
   if (p->mask_block_tokens < 0) return SDV2_ERR_INVALID_ARG;
@@ -1240,6 +1357,14 @@ int attn_fwd(const sdv2_attn_params* p, void* workspace, size_t workspace_bytes)
     a.split_h = a.split_t + third;
   }
 
+  if (p->q_norm_weight || p->q_inv_rms) {
+    // the raw q projection: normalised, then rotated, as it is loaded
+    if (!p->q_norm_weight || !p->q_inv_rms || !p->rope_freqs) return SDV2_ERR_INVALID_ARG;
+    if (!aligned16(p->q_norm_weight) || (reinterpret_cast<uintptr_t>(p->q_inv_rms) & 3)) return SDV2_ERR_INVALID_ARG;
+    a.q_norm_w = static_cast<const uint16_t*>(p->q_norm_weight);
+    a.q_inv_rms = p->q_inv_rms;
+  }
+
   a.q_blocks = (p->q_tokens + kQBlock - 1) / kQBlock;
   if (splits > 1) {
     const WorkspaceLayout w = workspace_layout(p->rows, p->q_tokens, p->heads, splits);
@@ -1253,7 +1378,9 @@ int attn_fwd(const sdv2_attn_params* p, void* workspace, size_t workspace_bytes)
   }
 
   hipStream_t stream = static_cast<hipStream_t>(p->stream);
-  const int64_t items = (int64_t)((p->q_tokens + kQTile - 1) / kQTile) * p->heads * p->rows * splits;
+  const int64_t nq_tiles = (p->q_tokens + kQTile - 1) / kQTile;
+  const int64_t items = ((int64_t)p->rows * p->heads / plan.group) *
+                        (nq_tiles * ((int64_t)(plan.group - plan.more) * plan.base + (int64_t)plan.more * (plan.base + 1)));
   if (items > (1 << 28)) return SDV2_ERR_INVALID_ARG;
   dim3 grid((unsigned)(8 * ((items + 7) / 8)));
   // The tile buffers (96 KB) or the epilogue staging (16 KB per wave) exceed the static limit:

@@ -235,7 +235,8 @@ int sdv2::attn_fwd_f32(const sdv2_attn_params* p) {
   if (!stride_ok(p->q_stride) || !stride_ok(p->k_stride) || !stride_ok(p->v_stride) || !stride_ok(p->out_stride))
     return SDV2_ERR_INVALID_ARG;
   if (p->rows > 65535 || p->heads > 65535) return SDV2_ERR_INVALID_ARG;
-  if (p->rope_freqs) return SDV2_ERR_UNSUPPORTED;       // fp32 queries arrive rotated (the append returns them)
+  if (p->rope_freqs || p->q_norm_weight || p->q_inv_rms)
+    return SDV2_ERR_UNSUPPORTED;                        // fp32 queries arrive normalised and rotated (the append returns them)
   if (p->mask_block_tokens < 0) return SDV2_ERR_INVALID_ARG;
 
   AttnF32Args a{};

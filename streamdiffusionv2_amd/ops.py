@@ -109,6 +109,7 @@ def kv_append_rope(
     new_local_end: Optional[Sequence[int]] = None,
     qk_norm: Optional[Tuple[torch.Tensor, torch.Tensor, float]] = None,
     dst_start_override: Optional[torch.Tensor] = None,
+    q_inv_rms: Optional[torch.Tensor] = None,
 ) -> Optional[torch.Tensor]:
     """RoPE q and k, write k' and v into the cache at ``dst_starts`` and store
     the new end indices.  Returns the roped query (``q_out`` or a new tensor).
@@ -119,7 +120,10 @@ def kv_append_rope(
 
     ``qk_norm`` = (q weight, k weight, eps) folds the WanRMSNorm of the
     projection outputs in (wan_base/modules/model.py:70-86): q and k are then
-    the raw projection outputs.
+    the raw projection outputs.  With ``q_inv_rms`` (float32 [B, S] on the
+    device) the kernel stores 1 / rms of every q token there and writes NO
+    rotated query (returns None): :func:`swa_attention` takes the raw q with
+    ``q_norm=(q weight, q_inv_rms)`` and normalises and rotates it itself.
 
     ``freqs_table`` is :func:`device_freqs` output.  Rows are processed in
     groups of at most 16 per launch.
@@ -131,7 +135,13 @@ def kv_append_rope(
         if t is not None and t.dtype != k.dtype:
             raise RuntimeError(f"dtype mismatch: {t.dtype} vs {k.dtype}")
     rows, tokens, heads, _ = k.shape
-    if q is not None and q_out is None:
+    if q_inv_rms is not None:
+        if qk_norm is None or q is None or q_out is not None:
+            raise RuntimeError("q_inv_rms goes with qk_norm and q, and replaces q_out")
+        if q_inv_rms.dtype != torch.float32 or q_inv_rms.numel() != rows * tokens or not q_inv_rms.is_contiguous() \
+                or q_inv_rms.device != dev:
+            raise RuntimeError(f"q_inv_rms must be a contiguous float32 tensor of {rows} x {tokens} elements on {dev}")
+    elif q is not None and q_out is None:
         q_out = torch.empty((rows, tokens, heads, HEAD_DIM), dtype=q.dtype, device=dev)
     for name, t in (("q", q), ("v", v), ("q_out", q_out)):
         if t is not None and tuple(t.shape) != tuple(k.shape):
@@ -161,7 +171,10 @@ def kv_append_rope(
             sl = slice(r0, r1)
             if q is not None:
                 p.q_in, p.q_in_stride = q[sl].data_ptr(), _stride3(q, "q")
-                p.q_out, p.q_out_stride = q_out[sl].data_ptr(), _stride3(q_out, "q_out")
+                if q_out is not None:
+                    p.q_out, p.q_out_stride = q_out[sl].data_ptr(), _stride3(q_out, "q_out")
+                else:
+                    p.q_inv_rms = q_inv_rms.data_ptr() + 4 * r0 * tokens
             p.k_in, p.k_in_stride = k[sl].data_ptr(), _stride3(k, "k")
             p.v_in, p.v_in_stride = v[sl].data_ptr(), _stride3(v, "v")
             p.k_cache, p.k_cache_stride = k_cache[sl].data_ptr(), _stride3(k_cache, "k_cache")
@@ -327,6 +340,7 @@ def swa_attention(
     mask_block_tokens: int = 0,
     static_scratch: bool = False,
     rope: Optional[Tuple[torch.Tensor, Sequence[int], Sequence[int]]] = None,
+    q_norm: Optional[Tuple[torch.Tensor, torch.Tensor]] = None,
 ) -> torch.Tensor:
     """out[b] = softmax(q[b] k_cache[b,:seq_lens[b]]^T * scale) v_cache[b,:seq_lens[b]].
 
@@ -334,6 +348,8 @@ def swa_attention(
     row): q is the query BEFORE RoPE and is rotated inside the kernel exactly as
     :func:`kv_append_rope` would have rotated it (S must be whole frames).  A
     caller-owned ``workspace`` must come from :func:`new_workspace` (zero-filled).
+    With ``q_norm`` = (q norm weight, q_inv_rms from :func:`kv_append_rope`) as
+    well, q is the raw q projection and is RMS-normalised before the rotation.
 
     ``static_scratch`` takes the library's allocation-free entry point
     (``sdv2_swa_attn_fwd_static``): partial results of a split call go to device
@@ -409,6 +425,16 @@ def swa_attention(
         p.rope_freqs, p.rope_freq_rows = table.data_ptr(), table.shape[0]
         p.rope_grid_h, p.rope_grid_w = int(grid_hw[0]), int(grid_hw[1])
         p.rope_start_frame = C.cast(frames, C.POINTER(C.c_int64))
+    if q_norm is not None:
+        weight, inv_rms = q_norm
+        if rope is None:
+            raise RuntimeError("q_norm needs rope=: the kernel normalises the raw query, then rotates it")
+        if weight.dtype != q.dtype or weight.numel() != heads * HEAD_DIM or not weight.is_contiguous() or weight.device != dev:
+            raise RuntimeError(f"the q norm weight must be a contiguous {q.dtype} tensor of {heads * HEAD_DIM} elements on {dev}")
+        if inv_rms.dtype != torch.float32 or inv_rms.numel() != rows * q_tokens or not inv_rms.is_contiguous() \
+                or inv_rms.device != dev:
+            raise RuntimeError(f"q_inv_rms must be a contiguous float32 tensor of {rows} x {q_tokens} elements on {dev}")
+        p.q_norm_weight, p.q_inv_rms = weight.data_ptr(), inv_rms.data_ptr()
     with torch.cuda.device(dev):
         if static_scratch:
             _capi.check(lib.sdv2_swa_attn_fwd_static(C.byref(p)), "sdv2_swa_attn_fwd_static")
@@ -611,11 +637,16 @@ class LayerLauncher:
         self.lib = _capi.lib()
         # The query is rotated where it is consumed, inside the attention kernel,
         # so the append moves K and V only.  With the q / k norm folded into the
-        # append (which needs whole tokens of q) or on request, the append rotates
-        # q as well and hands the attention the rotated copy in ``roped_q``.
-        self.rope_in_attention = bool(rope_in_attention) and qk_norm is None
+        # append the append still reads q - the norm needs the sum of squares of
+        # whole tokens - but only leaves 1 / rms per token (``q_inv_rms``) for the
+        # attention kernel, which normalises and rotates.  On request
+        # (rope_in_attention=False) the append rotates q as well and hands the
+        # attention the rotated copy in ``roped_q``.
+        self.rope_in_attention = bool(rope_in_attention)
         self.roped_q = None if self.rope_in_attention else torch.empty(
             (rows, tokens, heads, HEAD_DIM), dtype=torch.bfloat16, device=dev)
+        self.q_inv_rms = torch.empty((rows, tokens), dtype=torch.float32, device=dev) \
+            if self.rope_in_attention and qk_norm is not None else None
         self.sf = (C.c_int64 * rows)()
         self.ds = (C.c_int64 * rows)()
         self.ng = (C.c_int64 * rows)()
@@ -627,6 +658,9 @@ class LayerLauncher:
         if not self.rope_in_attention:
             ap.q_in_stride = _stride3(q_like, "q")
             ap.q_out, ap.q_out_stride = self.roped_q.data_ptr(), _stride3(self.roped_q, "q_out")
+        elif self.q_inv_rms is not None:
+            ap.q_in_stride = _stride3(q_like, "q")
+            ap.q_inv_rms = self.q_inv_rms.data_ptr()
         ap.k_cache, ap.k_cache_stride = k_cache.data_ptr(), _stride3(k_cache, "k_cache")
         ap.v_cache, ap.v_cache_stride = v_cache.data_ptr(), _stride3(v_cache, "v_cache")
         ap.freqs, ap.freq_rows = freqs_table.data_ptr(), freqs_table.shape[0]
@@ -654,6 +688,8 @@ class LayerLauncher:
             at.rope_freqs, at.rope_freq_rows = freqs_table.data_ptr(), freqs_table.shape[0]
             at.rope_grid_h, at.rope_grid_w = int(grid[1]), int(grid[2])
             at.rope_start_frame = C.cast(self.sf, C.POINTER(C.c_int64))
+            if self.q_inv_rms is not None:
+                at.q_norm_weight, at.q_inv_rms = qk_norm[0].data_ptr(), self.q_inv_rms.data_ptr()
         else:
             at.q, at.q_stride = self.roped_q.data_ptr(), _stride3(self.roped_q, "q")
         at.k_cache, at.k_stride = k_cache.data_ptr(), _stride3(k_cache, "k_cache")
@@ -699,6 +735,8 @@ class LayerLauncher:
         ap.k_in, ap.v_in = k.data_ptr(), v.data_ptr()
         if self.rope_in_attention:
             at.q = q.data_ptr()
+            if self.q_inv_rms is not None:
+                ap.q_in = q.data_ptr()
         else:
             ap.q_in = q.data_ptr()
         stream = _stream_ptr(self.dev)

@@ -68,10 +68,10 @@ int main(void) {
   expect("relayout index without source", sdv2_cache_relayout(&rl), SDV2_ERR_INVALID_ARG);
 
   /* struct layouts, for the bindings to compare themselves with */
-  printf("layout sdv2_append_params size=%zu stream=%zu dst_start_override=%zu\n", sizeof(sdv2_append_params),
-         offsetof(sdv2_append_params, stream), offsetof(sdv2_append_params, dst_start_override));
-  printf("layout sdv2_attn_params size=%zu stream=%zu dtype=%zu\n", sizeof(sdv2_attn_params),
-         offsetof(sdv2_attn_params, stream), offsetof(sdv2_attn_params, dtype));
+  printf("layout sdv2_append_params size=%zu stream=%zu q_inv_rms=%zu\n", sizeof(sdv2_append_params),
+         offsetof(sdv2_append_params, stream), offsetof(sdv2_append_params, q_inv_rms));
+  printf("layout sdv2_attn_params size=%zu stream=%zu q_inv_rms=%zu\n", sizeof(sdv2_attn_params),
+         offsetof(sdv2_attn_params, stream), offsetof(sdv2_attn_params, q_inv_rms));
   printf("layout sdv2_sink_sim_params size=%zu stream=%zu planned_frame=%zu\n", sizeof(sdv2_sink_sim_params),
          offsetof(sdv2_sink_sim_params, stream), offsetof(sdv2_sink_sim_params, planned_frame));
   printf("layout sdv2_relayout_params size=%zu stream=%zu global_end_shift=%zu\n", sizeof(sdv2_relayout_params),

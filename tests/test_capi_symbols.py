@@ -200,8 +200,8 @@ def test_plain_c_caller(tmp_path):
     import ctypes as C
     import re
 
-    for c_name, binding, last in (("sdv2_append_params", _capi.AppendParams, "dst_start_override"),
-                                  ("sdv2_attn_params", _capi.AttnParams, "dtype"),
+    for c_name, binding, last in (("sdv2_append_params", _capi.AppendParams, "q_inv_rms"),
+                                  ("sdv2_attn_params", _capi.AttnParams, "q_inv_rms"),
                                   ("sdv2_sink_sim_params", _capi.SinkSimParams, "planned_frame"),
                                   ("sdv2_relayout_params", _capi.RelayoutParams, "global_end_shift")):
         m = re.search(rf"layout {c_name} size=(\d+) stream=(\d+) {last}=(\d+)", run.stdout)

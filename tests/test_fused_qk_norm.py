@@ -160,6 +160,73 @@ def test_fused_norm_append(gpu_device, heads, dtype):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("heads", [12, 40, 5, 64])
+def test_attention_normalises_and_rotates_the_raw_query_itself(gpu_device, heads):
+    """With q_inv_rms the fused append writes no rotated query: it leaves
+    1 / rms per token, and the attention kernel normalises and rotates the raw
+    q projection while it loads it.  Same roundings in the same order, so cache
+    bits, 1 / rms and the attention output are those of the path that goes
+    through the rotated copy."""
+    from streamdiffusionv2_amd import ops, ring, rope
+
+    print(f"q norm inside the attention kernel: heads={heads}", flush=True)
+    torch.manual_seed(11 + heads)
+    rows, grid, cap = 2, (2, 5, 6), 240
+    S, eps = 60, 1e-6
+    dev = gpu_device
+    q = (torch.randn(rows, S, heads, 128) * 1.7).bfloat16().to(dev)
+    k = (torch.randn(rows, S, heads, 128) * 0.6).bfloat16().to(dev)
+    v = torch.randn(rows, S, heads, 128).bfloat16().to(dev)
+    wq = (torch.rand(heads * 128) + 0.5).bfloat16().to(dev)
+    wk = (torch.rand(heads * 128) + 0.5).bfloat16().to(dev)
+    start_frames, dst = [3, 9], [60, 120]
+    table = ops.device_freqs(rope.build_freqs(), dev)
+    results = []
+    for leave_inv_rms in (False, True):
+        caches = ring.new_kv_cache(1, 1, cap, heads, 1, device=dev)
+        ring.replicate_for_stream_batch(caches, rows)
+        cache = caches[0]
+        for name in ("k", "v"):                    # older keys for the chunk to attend to
+            cache[name].copy_(torch.randn(rows, cap, heads, 128, generator=torch.Generator().manual_seed(5)).bfloat16())
+        inv = torch.empty(rows, S, dtype=torch.float32, device=dev) if leave_inv_rms else None
+        roped = ops.kv_append_rope(q, k, v, cache["k"], cache["v"], table, grid, start_frames, dst,
+                                   qk_norm=(wq, wk, eps), q_inv_rms=inv)
+        if leave_inv_rms:
+            assert roped is None
+            out = ops.swa_attention(q, cache["k"], cache["v"], None, rope=(table, grid[1:], start_frames), q_norm=(wq, inv))
+        else:
+            out = ops.swa_attention(roped, cache["k"], cache["v"], None)
+        torch.cuda.synchronize()
+        results.append((out.cpu(), cache["k"].cpu(), cache["v"].cpu(), inv))
+    (out0, k0, v0, _), (out1, k1, v1, inv) = results
+    assert torch.equal(k0.view(torch.int16), k1.view(torch.int16)) and torch.equal(v0.view(torch.int16), v1.view(torch.int16))
+    assert torch.equal(out0.view(torch.int16), out1.view(torch.int16))
+    want_inv = torch.rsqrt(q.float().cpu().flatten(2).pow(2).mean(-1) + eps)
+    assert (inv.cpu() - want_inv).abs().max().item() <= 2e-6 * want_inv.abs().max().item()
+
+
+@pytest.mark.gpu
+def test_q_norm_argument_errors(gpu_device):
+    from streamdiffusionv2_amd import ops, rope
+
+    table = ops.device_freqs(rope.build_freqs(), gpu_device)
+    x = torch.zeros(1, 6, 2, 128, dtype=torch.bfloat16, device=gpu_device)
+    cache = torch.zeros(1, 12, 2, 128, dtype=torch.bfloat16, device=gpu_device)
+    w = torch.ones(256, dtype=torch.bfloat16, device=gpu_device)
+    inv = torch.ones(1, 6, dtype=torch.float32, device=gpu_device)
+    with pytest.raises(RuntimeError):       # 1 / rms only exists with the norm
+        ops.kv_append_rope(x, x, x, cache, cache.clone(), table, (1, 2, 3), [0], [0], q_inv_rms=inv)
+    with pytest.raises(RuntimeError):       # one entry per token
+        ops.kv_append_rope(x, x, x, cache, cache.clone(), table, (1, 2, 3), [0], [0], qk_norm=(w, w, 1e-6), q_inv_rms=inv[:, :5])
+    with pytest.raises(RuntimeError):       # the kernel normalises, then rotates: it needs the table
+        ops.swa_attention(x, cache, cache, None, q_norm=(w, inv))
+    with pytest.raises(RuntimeError):
+        ops.swa_attention(x, cache, cache, None, rope=(table, (2, 3), [0]), q_norm=(w[:128], inv))
+    ops.swa_attention(x, cache, cache, None, rope=(table, (2, 3), [0]), q_norm=(w, inv))
+    torch.cuda.synchronize()
+
+
+@pytest.mark.gpu
 def test_module_with_and_without_fusion(gpu_device):
     from streamdiffusionv2_amd import ring, rope
     from streamdiffusionv2_amd.attention import CausalWanSelfAttention

@@ -79,6 +79,46 @@ def test_attention_exact_fallback_on_extreme_scores(gpu_device, kind, splits):
     _check(got.cpu(), want)
 
 
+@pytest.mark.parametrize("plan", [3 | (1 << 8), 1 | (1 << 8), 2 | (3 << 8), 4])
+def test_mixed_split_plans(gpu_device, plan):
+    """num_splits may ask for one key range more on some (row, head) pairs of
+    every XCD's share (bits 8-15): workgroups of two lengths, partial results
+    of two different counts in one launch.  Ragged lengths, rows of the last
+    query tile that do not exist."""
+    from streamdiffusionv2_amd import ops
+
+    torch.manual_seed(40 + plan)
+    rows, S, H, L = 4, 300, 8, 1500            # 32 pairs: four per XCD
+    q = torch.randn(rows, S, H, 128).bfloat16()
+    k = torch.randn(rows, L, H, 128).bfloat16()
+    v = torch.randn(rows, L, H, 128).bfloat16()
+    lens = [1500, 777, 64, 1201]
+    want = oracle.attention_fp32_reference(q, k, v, lens)
+    sl = torch.tensor(lens, dtype=torch.int32, device=gpu_device)
+    got = ops.swa_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), sl, num_splits=plan)
+    again = ops.swa_attention(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), sl, num_splits=plan)
+    torch.cuda.synchronize()
+    assert torch.equal(got, again)
+    _check(got.cpu(), want)
+
+
+def test_split_plans_the_library_refuses(gpu_device):
+    from streamdiffusionv2_amd import ops
+
+    q = torch.zeros(1, 64, 12, 128, dtype=torch.bfloat16, device=gpu_device)
+    kv = torch.zeros(1, 2048, 12, 128, dtype=torch.bfloat16, device=gpu_device)
+    with pytest.raises(RuntimeError):          # 12 pairs do not divide over the eight XCDs
+        ops.swa_attention(q, kv, kv, None, num_splits=2 | (1 << 8))
+    q16 = torch.zeros(2, 64, 8, 128, dtype=torch.bfloat16, device=gpu_device)
+    kv16 = torch.zeros(2, 2048, 8, 128, dtype=torch.bfloat16, device=gpu_device)
+    with pytest.raises(RuntimeError):          # two pairs per XCD: at most one of them can take one range more
+        ops.swa_attention(q16, kv16, kv16, None, num_splits=2 | (2 << 8))
+    with pytest.raises(RuntimeError):
+        ops.swa_attention(q16, kv16, kv16, None, num_splits=1 << 16)
+    ops.swa_attention(q16, kv16, kv16, None, num_splits=2 | (1 << 8))
+    torch.cuda.synchronize()
+
+
 def test_attention_tiny_sequences(gpu_device):
     from streamdiffusionv2_amd import ops
 
