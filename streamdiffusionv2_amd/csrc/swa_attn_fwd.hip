@@ -88,8 +88,11 @@ constexpr int kKTile = 64;
 constexpr int kTileBytes = kKTile * kD * 2; // 16 KB per matrix
 constexpr int kStages = 3;
 constexpr int kStageBytes = 16384;          // epilogue staging per wave: 32 rows x 512 B
-constexpr int kLdsBytes = 2 * kStages * kTileBytes > kWaves * kStageBytes ? 2 * kStages * kTileBytes
+// Two flag words of the workgroup sit behind the tile buffers and the staging
+// areas, so that setting and reading them needs no barrier of its own.
+constexpr int kLdsFlags = 2 * kStages * kTileBytes > kWaves * kStageBytes ? 2 * kStages * kTileBytes
                                                                          : kWaves * kStageBytes;
+constexpr int kLdsBytes = kLdsFlags + 256;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kCuSlots = 256;               // one workgroup per CU
 constexpr int kMaxDevices = 64;
@@ -650,6 +653,8 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   lds_char* lds = (lds_char*)smem;
 
+  lds_int* flags = reinterpret_cast<lds_int*>(lds + kLdsFlags);
+
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -749,6 +754,7 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
       *reinterpret_cast<__attribute__((address_space(3))) u32x4*>(lds + kLdsV(2) + tid * 16) = zero;
       *reinterpret_cast<__attribute__((address_space(3))) u32x4*>(lds + kLdsV(2) + (kThreads + tid) * 16) = zero;
     }
+    if (tid == 0) flags[0] = 0;       // "a wave found an unsafe row sum": read behind the barrier that ends the loop
   }
 
   // ---- this lane's query row -------------------------------------------------
@@ -944,20 +950,19 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
       }
     }
 
-    // Did any wave of the workgroup see an unsafe row sum?  (LDS is free now.)
+    // Did any wave of the workgroup see an unsafe row sum?  One barrier: behind it every wave is done
+    // with the K / V buffers (the epilogue stages its output there) and the flag, cleared before the
+    // loop, holds every wave's word.
+    if (unsafe && lane == 0) flags[0] = 1;
     __syncthreads();
-    if (tid == 0) *reinterpret_cast<lds_int*>(lds) = 0;
-    __syncthreads();
-    if (unsafe && lane == 0) *reinterpret_cast<lds_int*>(lds) = 1;
-    __syncthreads();
-    const int redo = *reinterpret_cast<lds_int*>(lds);
+    const int redo = flags[0];
     if (redo)
       exact_pass(c, qf, oacc, m_run, l_run, unsafe, kbase, vbase, k_tok_bytes, v_tok_bytes, k_ld, v_ld, tile_begin, n,
                  seq, lds_addr0, lds, wave_u, lane);
   }
 
   // ---- epilogue ---------------------------------------------------------------
-  __syncthreads();                    // every wave is done with the K / V buffers
+  // (every wave is done with the K / V buffers: the barrier above, or the last one of the exact pass)
   const int block = qtile * kWaves + wave;              // this wave's 32-row block within the (row, head)
   float l_tot = half_sum(l_run);
   float inv = l_tot > 0.f ? 1.0f / l_tot : 0.f;
@@ -1013,11 +1018,10 @@ void swa_attn_fwd_kernel(const AttnKernelArgs a) {
       const int drawn = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       const int last = drawn == nsplits - 1;
       if (last) __hip_atomic_store(ticket, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      *reinterpret_cast<lds_int*>(lds) = last;
+      flags[1] = last;
     }
     __syncthreads();
-    if (*reinterpret_cast<lds_int*>(lds) == 0 || idle) return;
-    __syncthreads();                  // (the flag word lies in wave 0's staging area)
+    if (flags[1] == 0 || idle) return;
 
     // combine: out = sum_s 2^(lse_s - LSE) O_s over the ranges in their fixed
     // order (every range, this workgroup's own included, as it lies in memory:
