@@ -70,6 +70,7 @@ struct SinkSimKernelArgs {
   int64_t* dst_override;                    // [rows] or null: slot start for the append that follows
   uint32_t override_rows;                   // bit i: row i is about to evict, so a refresh moves its write
   int32_t tokens, heads, grid_w, sink_frames;
+  int32_t first_matrix;                     // matrices below this one are not summed in this call: the grid leaves them out
   int32_t split_t, split_h, pairs;
   float threshold;
   int64_t start_frame[SDV2_MAX_ROWS];
@@ -85,6 +86,72 @@ __device__ __forceinline__ void store_coherent(float* p, float x) {
 __device__ __forceinline__ float load_coherent(const float* p) {
   return __uint_as_float(
       __hip_atomic_load(reinterpret_cast<const uint32_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+
+// The token sums of four neighbouring columns, all kTokenSplits ranges (512
+// bytes apart): 16-byte device-coherent loads, which have no spelling in the
+// language.  Issue and wait are ONE asm statement: between a load's issue and
+// its return the compiler believes the destination registers hold the value and
+// is free to copy or reuse them.
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+__device__ __forceinline__ void load_coherent_ranges(const float* base, f32x4 (&w)[8]) {
+  static_assert(kTokenSplits == 8, "eight ranges per statement");
+  asm volatile(
+      "global_load_dwordx4 %0, %8, off sc1\n\t"
+      "global_load_dwordx4 %1, %8, off offset:512 sc1\n\t"
+      "global_load_dwordx4 %2, %8, off offset:1024 sc1\n\t"
+      "global_load_dwordx4 %3, %8, off offset:1536 sc1\n\t"
+      "global_load_dwordx4 %4, %8, off offset:2048 sc1\n\t"
+      "global_load_dwordx4 %5, %8, off offset:2560 sc1\n\t"
+      "global_load_dwordx4 %6, %8, off offset:3072 sc1\n\t"
+      "global_load_dwordx4 %7, %8, off offset:3584 sc1\n\t"
+      "s_waitcnt vmcnt(0)"
+      : "=&v"(w[0]), "=&v"(w[1]), "=&v"(w[2]), "=&v"(w[3]), "=&v"(w[4]), "=&v"(w[5]), "=&v"(w[6]), "=&v"(w[7])
+      : "v"(base)
+      : "memory");
+}
+// the same for two groups of four columns in one trip
+__device__ __forceinline__ void load_coherent_ranges2(const float* base0, const float* base1, f32x4 (&w0)[8], f32x4 (&w1)[8]) {
+  asm volatile(
+      "global_load_dwordx4 %0, %16, off sc1\n\t"
+      "global_load_dwordx4 %1, %16, off offset:512 sc1\n\t"
+      "global_load_dwordx4 %2, %16, off offset:1024 sc1\n\t"
+      "global_load_dwordx4 %3, %16, off offset:1536 sc1\n\t"
+      "global_load_dwordx4 %4, %16, off offset:2048 sc1\n\t"
+      "global_load_dwordx4 %5, %16, off offset:2560 sc1\n\t"
+      "global_load_dwordx4 %6, %16, off offset:3072 sc1\n\t"
+      "global_load_dwordx4 %7, %16, off offset:3584 sc1\n\t"
+      "global_load_dwordx4 %8, %17, off sc1\n\t"
+      "global_load_dwordx4 %9, %17, off offset:512 sc1\n\t"
+      "global_load_dwordx4 %10, %17, off offset:1024 sc1\n\t"
+      "global_load_dwordx4 %11, %17, off offset:1536 sc1\n\t"
+      "global_load_dwordx4 %12, %17, off offset:2048 sc1\n\t"
+      "global_load_dwordx4 %13, %17, off offset:2560 sc1\n\t"
+      "global_load_dwordx4 %14, %17, off offset:3072 sc1\n\t"
+      "global_load_dwordx4 %15, %17, off offset:3584 sc1\n\t"
+      "s_waitcnt vmcnt(0)"
+      : "=&v"(w0[0]), "=&v"(w0[1]), "=&v"(w0[2]), "=&v"(w0[3]), "=&v"(w0[4]), "=&v"(w0[5]), "=&v"(w0[6]), "=&v"(w0[7]),
+        "=&v"(w1[0]), "=&v"(w1[1]), "=&v"(w1[2]), "=&v"(w1[3]), "=&v"(w1[4]), "=&v"(w1[5]), "=&v"(w1[6]), "=&v"(w1[7])
+      : "v"(base0), "v"(base1)
+      : "memory");
+}
+
+// Sum over the 64 lanes of a wave without a trip through LDS per step: within
+// quads, rows of 16 lanes, then across the rows (the wave-wide broadcasts of
+// the data-parallel-primitive operand modes); lane 63 ends up with the total.
+__device__ __forceinline__ float wave_sum(float x) {
+  auto dpp = [](float v, auto ctrl_c, auto rows_c) {
+    constexpr int ctrl = decltype(ctrl_c)::value, rows = decltype(rows_c)::value;
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), ctrl, rows, 0xf, false));
+  };
+  using All = std::integral_constant<int, 0xf>;
+  x += dpp(x, std::integral_constant<int, 0xb1>{}, All{});      // quad_perm [1, 0, 3, 2]
+  x += dpp(x, std::integral_constant<int, 0x4e>{}, All{});      // quad_perm [2, 3, 0, 1]
+  x += dpp(x, std::integral_constant<int, 0x141>{}, All{});     // row_half_mirror
+  x += dpp(x, std::integral_constant<int, 0x140>{}, All{});     // row_mirror
+  x += dpp(x, std::integral_constant<int, 0x142>{}, std::integral_constant<int, 0xa>{});   // row_bcast15 into rows 1, 3
+  x += dpp(x, std::integral_constant<int, 0x143>{}, std::integral_constant<int, 0xc>{});   // row_bcast31 into rows 2, 3
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 63));
 }
 
 // matrices of a row: sink K frames, sink V frames, new K, new V
@@ -128,35 +195,35 @@ __device__ __forceinline__ void decide(const SinkSimKernelArgs& a, int row) {
   const int width = a.heads * 128;
   const float inv_tokens = 1.0f / static_cast<float>(a.tokens);
   constexpr float kEps = 1e-8f;             // torch.cosine_similarity default
-  // column i of this thread, and its weight (0 past the width)
+  // Column i of this thread, and its weight (0 past the width).  Columns come
+  // in groups of four neighbours (4 * thread .. 4 * thread + 3, then 4 * kThreads
+  // further on), so that the token sums of a group arrive in 16-byte accesses;
+  // a group past the width is clamped to the last group and weighted with zero.
+  static_assert(kCols % 4 == 0, "columns are owned in groups of four");
+  auto raw_col = [&](int i) { return 4 * static_cast<int>(threadIdx.x) + (i & 3) + (i >> 2) * 4 * kThreads; };
   auto col = [&](int i) {
-    const int c = static_cast<int>(threadIdx.x) + i * kThreads;
-    return c < width ? c : width - 1;
+    const int c = raw_col(i);
+    return c < width ? c : width - 4 + (i & 3);
   };
-  auto live = [&](int i) { return static_cast<int>(threadIdx.x) + i * kThreads < width ? 1.f : 0.f; };
+  // where the eight ranges' sums of the column group that starts at column i of this thread begin
+  auto ranges_of = [&](const float* p, int i) { return p + (col(i) >> 7) * (kTokenSplits * 128) + (col(i) & 127); };
+  auto live = [&](int i) { return raw_col(i) < width ? 1.f : 0.f; };
   // means of matrix m at this thread's columns: the token ranges in order and
   // the rounding of a stored mean, or the mean kept from an earlier call.  The
   // token sums are fetched for eight columns at a time (64 loads in flight).
   auto means = [&](int m, float (&out)[kCols]) {
     if (summed_now(a, row, m)) {
       const float* p = sums_of(a, row, m);
-      constexpr int kChunk = 8;
 #pragma unroll
-      for (int i0 = 0; i0 < kCols; i0 += kChunk) {
-        float part[kChunk][kTokenSplits];
+      for (int i0 = 0; i0 < kCols; i0 += 4) {
+        f32x4 part[kTokenSplits];
+        load_coherent_ranges(ranges_of(p, i0), part);
 #pragma unroll
-        for (int i = 0; i < kChunk; ++i)
-#pragma unroll
-          for (int j = 0; j < kTokenSplits; ++j)
-            if (i0 + i < kCols)
-              part[i][j] = load_coherent(p + ((col(i0 + i) >> 7) * kTokenSplits + j) * 128 + (col(i0 + i) & 127));
-#pragma unroll
-        for (int i = 0; i < kChunk; ++i) {
-          if (i0 + i >= kCols) continue;
+        for (int e = 0; e < 4; ++e) {
           float sum = 0.f;
 #pragma unroll
-          for (int j = 0; j < kTokenSplits; ++j) sum += part[i][j];
-          out[i0 + i] = round_to_storage<T>(sum * inv_tokens);
+          for (int j = 0; j < kTokenSplits; ++j) sum += part[j][e];
+          out[i0 + e] = round_to_storage<T>(sum * inv_tokens);
         }
       }
       if (a.kept && m < 2 * sink) {
@@ -173,9 +240,7 @@ __device__ __forceinline__ void decide(const SinkSimKernelArgs& a, int row) {
   // this wave's share of four sums, in a fixed order, parked in LDS
   auto park = [&](int slot, float (&x)[4]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int off = 32; off > 0; off >>= 1) x[i] += __shfl_xor(x[i], off, 64);
+    for (int i = 0; i < 4; ++i) x[i] = wave_sum(x[i]);
     if ((threadIdx.x & 63) == 0)
 #pragma unroll
       for (int i = 0; i < 4; ++i) wave_part[slot][threadIdx.x >> 6][i] = x[i];
@@ -204,25 +269,21 @@ __device__ __forceinline__ void decide(const SinkSimKernelArgs& a, int row) {
   fetch_frames(0);
   float k_new[kCols], v_new[kCols];
   if constexpr (kCols <= 8) {
-    // few enough columns per thread that the token sums of both new matrices
-    // fit the registers at once: one trip to memory instead of two
-    float part[2][kCols][kTokenSplits];
+    // two column groups per thread: all the token sums of a new matrix come in one trip to memory
+    static_assert(kCols == 8, "two column groups per thread");
+    f32x4 part[2][2][kTokenSplits];          // matrix, column group, token range
 #pragma unroll
     for (int m = 0; m < 2; ++m) {
       const float* p = sums_of(a, row, 2 * sink + m);
-#pragma unroll
-      for (int i = 0; i < kCols; ++i)
-#pragma unroll
-        for (int j = 0; j < kTokenSplits; ++j)
-          part[m][i][j] = load_coherent(p + ((col(i) >> 7) * kTokenSplits + j) * 128 + (col(i) & 127));
+      load_coherent_ranges2(ranges_of(p, 0), ranges_of(p, 4), part[m][0], part[m][1]);
     }
 #pragma unroll
     for (int i = 0; i < kCols; ++i) {
       float sum_k = 0.f, sum_v = 0.f;
 #pragma unroll
       for (int j = 0; j < kTokenSplits; ++j) {
-        sum_k += part[0][i][j];
-        sum_v += part[1][i][j];
+        sum_k += part[0][i >> 2][j][i & 3];
+        sum_v += part[1][i >> 2][j][i & 3];
       }
       k_new[i] = round_to_storage<T>(sum_k * inv_tokens);
       v_new[i] = round_to_storage<T>(sum_v * inv_tokens);
@@ -302,8 +363,9 @@ __device__ __forceinline__ void decide(const SinkSimKernelArgs& a, int row) {
   }
 }
 
-// grid (heads, 2*sink+2, rows * kTokenSplits): one workgroup sums one head's
-// 128 columns of one frame over one eighth of its tokens.  (One workgroup per
+// grid (heads, matrices summed in this call, rows * kTokenSplits): one workgroup sums one head's
+// 128 columns of one frame over one eighth of its tokens.  (With every sink
+// frame's mean kept, the matrices are the new K and V alone: first_matrix.)  (One workgroup per
 // frame and head would leave most of the chip idle: 96 workgroups for three
 // sink frames of twelve heads.)  Then it draws its row's ticket, after its
 // sums have been acknowledged by memory; the workgroup that draws the last one
@@ -317,7 +379,7 @@ void sink_similarity_kernel(const SinkSimKernelArgs a) {
   const int lane = threadIdx.x & (kLanesPerRow - 1);
   const int tl = threadIdx.x >> 4;
   const int head = blockIdx.x;
-  const int m = blockIdx.y;
+  const int m = blockIdx.y + a.first_matrix;
   const int row = blockIdx.z / kTokenSplits;
   const int split = blockIdx.z - row * kTokenSplits;
   const int sink = a.sink_frames;
@@ -334,9 +396,17 @@ void sink_similarity_kernel(const SinkSimKernelArgs a) {
   const int per = (a.tokens + kTokenSplits - 1) / kTokenSplits;
   const int t_end = (split + 1) * per < a.tokens ? (split + 1) * per : a.tokens;
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  constexpr int kUnroll = 4;
+  // A token lane walks every sixteenth token of the range.  The range is short
+  // (195 tokens of a 1560-token frame: 12 or 13 per lane) and every trip to
+  // memory costs the same few microseconds whatever it carries, so a lane asks
+  // for up to kFlight of its tokens at once; past the end of the range it asks
+  // for the last token again and leaves it out of the sum.  The order of the
+  // adds is the token order.
+  constexpr int kFlight = 16;
   if (is_new && is_k) {
-    // the new keys are rotated on the way in; four tokens per trip, loads (data and table) issued together
+    // the new keys are rotated on the way in; their table entries (four per lane and token) are fetched for
+    // half a flight at a time, which is what the registers hold beside the tokens themselves
+    constexpr int kHalf = kFlight / 2;
     auto rotation = [&](int t, double2 (&cs)[4]) {
       const int hi = t / a.grid_w;
       sdv2::load_rotation(a.freqs, a.pairs, a.split_t, a.split_h, lane, a.start_frame[row], hi, t - hi * a.grid_w, cs);
@@ -344,51 +414,49 @@ void sink_similarity_kernel(const SinkSimKernelArgs a) {
     // with the norm folded in: the key as the append will normalise it (same two roundings)
     sdv2::Vec8<T> weight;
     if (a.k_norm_w) weight = sdv2::Vec8<T>::load(static_cast<const T*>(a.k_norm_w) + head * 128 + lane * 8);
-    auto normalised = [&](const sdv2::Vec8<T>& x, int t) {
-      return sdv2::normalise(x, a.inv_rms[static_cast<int64_t>(row) * a.tokens + t], weight);
-    };
-    int t = split * per + tl;
-    for (; t + (kUnroll - 1) * kTokenLanes < t_end; t += kUnroll * kTokenLanes) {
-      sdv2::Vec8<T> x[kUnroll];
-      double2 cs[kUnroll][4];
+    for (int t0 = split * per + tl; t0 < t_end; t0 += kFlight * kTokenLanes) {
+      sdv2::Vec8<T> x[kFlight];
+      float r[kFlight];
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-        x[u] = sdv2::Vec8<T>::load(base + (t + u * kTokenLanes) * st.token);
-        rotation(t + u * kTokenLanes, cs[u]);
+      for (int u = 0; u < kFlight; ++u) {
+        const int t = t0 + u * kTokenLanes < t_end ? t0 + u * kTokenLanes : t_end - 1;
+        x[u] = sdv2::Vec8<T>::load(base + t * st.token);
+        r[u] = a.k_norm_w ? a.inv_rms[static_cast<int64_t>(row) * a.tokens + t] : 1.0f;
       }
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) {
-        if (a.k_norm_w) x[u] = normalised(x[u], t + u * kTokenLanes);
-        const sdv2::Vec8<T> y = sdv2::rotate(x[u], cs[u]);
+      for (int half = 0; half < 2; ++half) {
+        if (t0 + half * kHalf * kTokenLanes >= t_end) break;
+        double2 cs[kHalf][4];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] += static_cast<float>(y.get(i));
+        for (int u = 0; u < kHalf; ++u) {
+          const int t = t0 + (half * kHalf + u) * kTokenLanes;
+          rotation(t < t_end ? t : t_end - 1, cs[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < kHalf; ++u) {
+          if (t0 + (half * kHalf + u) * kTokenLanes < t_end) {
+            sdv2::Vec8<T> xx = x[half * kHalf + u];
+            if (a.k_norm_w) xx = sdv2::normalise(xx, r[half * kHalf + u], weight);
+            const sdv2::Vec8<T> y = sdv2::rotate(xx, cs[u]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] += static_cast<float>(y.get(i));
+          }
+        }
       }
-    }
-    for (; t < t_end; t += kTokenLanes) {
-      double2 cs[4];
-      rotation(t, cs);
-      sdv2::Vec8<T> x = sdv2::Vec8<T>::load(base + t * st.token);
-      if (a.k_norm_w) x = normalised(x, t);
-      const sdv2::Vec8<T> y = sdv2::rotate(x, cs);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] += static_cast<float>(y.get(i));
     }
   } else {
-    // four tokens per trip, their loads issued together; the order of the adds is the token order
-    int t = split * per + tl;
-    for (; t + (kUnroll - 1) * kTokenLanes < t_end; t += kUnroll * kTokenLanes) {
-      sdv2::Vec8<T> x[kUnroll];
+    for (int t0 = split * per + tl; t0 < t_end; t0 += kFlight * kTokenLanes) {
+      sdv2::Vec8<T> x[kFlight];
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u) x[u] = sdv2::Vec8<T>::load(base + (t + u * kTokenLanes) * st.token);
+      for (int u = 0; u < kFlight; ++u) {
+        const int t = t0 + u * kTokenLanes < t_end ? t0 + u * kTokenLanes : t_end - 1;
+        x[u] = sdv2::Vec8<T>::load(base + t * st.token);
+      }
 #pragma unroll
-      for (int u = 0; u < kUnroll; ++u)
+      for (int u = 0; u < kFlight; ++u)
+        if (t0 + u * kTokenLanes < t_end)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] += static_cast<float>(x[u].get(i));
-    }
-    for (; t < t_end; t += kTokenLanes) {
-      const sdv2::Vec8<T> x = sdv2::Vec8<T>::load(base + t * st.token);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) acc[i] += static_cast<float>(x.get(i));
+          for (int i = 0; i < 8; ++i) acc[i] += static_cast<float>(x[u].get(i));
     }
   }
 #pragma unroll
@@ -532,7 +600,12 @@ extern "C" int sdv2_sink_similarity(const sdv2_sink_sim_params* p) {
 
   hipStream_t stream = static_cast<hipStream_t>(p->stream);
   const dim3 block(kThreads);
-  const dim3 grid(p->heads, 2 * p->sink_frames + 2, p->rows * kTokenSplits);
+  // no frame of any row stale: the grid holds the new chunk's two matrices only (workgroups that
+  // would find nothing to sum still cost their dispatch, and the ones that work start behind them)
+  bool any_stale = false;
+  for (int i = 0; i < p->rows; ++i) any_stale |= (a.stale[i] & ((1u << p->sink_frames) - 1u)) != 0;
+  a.first_matrix = any_stale ? 0 : 2 * p->sink_frames;
+  const dim3 grid(p->heads, 2 * p->sink_frames + 2 - a.first_matrix, p->rows * kTokenSplits);
   if (p->k_norm_weight) {
     const dim3 grid_rms((p->tokens + 3) / 4, 1, p->rows);
     const int steps = (p->heads + 3) / 4;
