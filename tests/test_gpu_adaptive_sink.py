@@ -438,6 +438,9 @@ def test_stream_with_refresh_production_shape(gpu_device, heads, seed, calls):
             assert torch.equal(cache[name].cpu().view(torch.int16), rec["cache_" + name].view(torch.int16)), (call, name)
         idx = torch.randperm(PROD_FT, generator=gen)[:32].sort().values
         want = oracle.attention_fp32_reference(rec["roped_q"][:, idx], rec["cache_k"], rec["cache_v"], rec["seq"])
+        # the recipe scales frames up to force clear decisions and the outputs
+        # grow with them: the unit-scale bounds (2e-2 / 2e-3) are taken relative
+        # to the largest output, as in the small-shape stream above
         unit = max(1.0, want.abs().max().item())
         err = (got[:, idx.to(gpu_device)].float().cpu() - want).abs()
         assert err.max().item() <= 2e-2 * unit and err.mean().item() <= 2e-3 * unit, call
