@@ -386,8 +386,9 @@ def module_path_section(args, w, headline_ms):
       inputs carry a scene direction that changes every eighth chunk, so the
       refresh check keeps the sink frames most of the time and replaces them,
       one per chunk, after a cut;
-    * ``module_forward``: whole forward() calls, with the four projection GEMMs
-      (vendor library) around the path.
+    * ``module_forward``: whole forward() calls, with the projection GEMMs
+      (vendor library; q, k and v as one launch, and as three for comparison)
+      around the path.
     Steady state, one chunk per step through every layer."""
     from streamdiffusionv2_amd import ring, workloads
     from streamdiffusionv2_amd.attention import CausalWanSelfAttention, RingKVPath
@@ -529,18 +530,25 @@ def module_path_section(args, w, headline_ms):
             mods[layer](x, None, grid, freqs, None, kv_cache=caches[layer], current_start=starts)
         state["call"] += 1
 
-    with torch.no_grad():
-        for _ in range(fill + args.warmup):
-            module_step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            module_step()
-        torch.cuda.synchronize()
-    per_layer = (time.perf_counter() - t0) * 1e3 / (args.steps * layers)
+    def timed():
+        with torch.no_grad():
+            for _ in range(fill + args.warmup):
+                module_step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                module_step()
+            torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / (args.steps * layers)
+
+    per_layer = timed()
+    for m in mods:
+        m.fuse_qkv_projection = False          # the reference's three launches, for comparison
+    per_layer_apart = timed()
     out["module_forward"] = {"ms_per_layer_call": per_layer, "ms_per_step": per_layer * w.layers, "layers_timed": layers,
-                             "what": "CausalWanSelfAttention.forward with its defaults: q / k / v / o projections "
-                                     "(vendor GEMMs) + the path; scaled to the layer count"}
+                             "ms_per_step_with_three_projection_launches": per_layer_apart * w.layers,
+                             "what": "CausalWanSelfAttention.forward with its defaults: q / k / v as one vendor GEMM "
+                                     "on the packed weights, the path, the o projection; scaled to the layer count"}
     return out
 
 

@@ -406,6 +406,20 @@ class CausalWanSelfAttention(nn.Module, RingKVPath):
         # separate torch modules before the path.
         self.fuse_qk_norm = True
 
+        # The q, k and v projections (causal_model.py:212-218 calls the three
+        # Linears one after the other) run as ONE vendor GEMM on the three
+        # weights laid end to end: at 1560 tokens x 1536 the three launches take
+        # 60 us and the one 26 us, with the same bits out (every output element
+        # is the same dot product over `dim`).  q, k and v are then strided views
+        # of one [B, S, 3 * dim] tensor, which the kernels of the path read as
+        # they are.  The packed copy of the weights (3 * dim * dim elements per
+        # layer) is rebuilt whenever a weight or bias has been replaced or
+        # written.  Only plain nn.Linear layers without forward hooks are packed
+        # (a wrapped layer or a hook gets the three calls it expects); False
+        # keeps the three launches and no copy.
+        self.fuse_qkv_projection = True
+        self._packed = None
+
         # ring state, same defaults as causal_model.py:177-179
         self.sink_size = 3
         self.adapt_sink_thr = -1
@@ -419,6 +433,51 @@ class CausalWanSelfAttention(nn.Module, RingKVPath):
         self.norm_k = WanRMSNorm(dim, eps=eps) if qk_norm else nn.Identity()
 
     # ------------------------------------------------------------------
+    def _packed_qkv(self):
+        """(weight [3 * dim, dim], bias [3 * dim] or None) of the q, k and v
+        Linears laid end to end, rebuilt when any of the six tensors has been
+        replaced (another tensor, dtype or device) or written in place."""
+        layers = (self.q, self.k, self.v)
+        for layer in layers:
+            # only plain Linears that nobody watches: a wrapped or replaced layer (an adapter, a quantised
+            # Linear) computes something else than x W^T + b, and a hook expects its layer to be called
+            if type(layer) is not nn.Linear or layer._forward_hooks or layer._forward_pre_hooks:
+                return None
+        tensors = [t for layer in layers for t in (layer.weight, layer.bias)]
+
+        def edits(t):
+            try:
+                return t._version
+            except RuntimeError:                   # a tensor made under inference_mode() counts no edits:
+                return -1                          # after writing such a weight in place, set _packed = None
+
+        key = tuple((t.data_ptr(), edits(t), t.dtype, t.device) if t is not None else None for t in tensors)
+        packed = self._packed
+        if packed is None or packed[0] != key:
+            with torch.no_grad():
+                weight = torch.cat([layer.weight.detach() for layer in layers], 0)
+                biases = [layer.bias for layer in layers]
+                bias = None
+                if all(b is not None for b in biases):
+                    bias = torch.cat([b.detach() for b in biases], 0)
+                elif any(b is not None for b in biases):
+                    return None                    # mixed: keep the three launches
+            packed = (key, weight, bias)
+            self._packed = packed
+        return packed[1], packed[2]
+
+    def project_qkv(self, x):
+        """The three projections of x [B, S, dim] -> q, k, v, each [B, S, dim]
+        (views of one tensor when they come out of one GEMM)."""
+        import torch.nn.modules.module as _hooks
+        watched = _hooks._global_forward_hooks or _hooks._global_forward_pre_hooks
+        packed = self._packed_qkv() if self.fuse_qkv_projection and not torch.is_grad_enabled() and not watched else None
+        if packed is None:
+            return self.q(x), self.k(x), self.v(x)
+        y = nn.functional.linear(x, packed[0], packed[1])
+        d = self.dim
+        return y[..., :d], y[..., d:2 * d], y[..., 2 * d:]
+
     def forward(
         self,
         x,
@@ -440,16 +499,17 @@ class CausalWanSelfAttention(nn.Module, RingKVPath):
                 "training path (causal_model.py:220-249) is out of scope"
             )
         b, s, n, d = *x.shape[:2], self.num_heads, self.head_dim
-        v = self.v(x).view(b, s, n, d)
+        q, k, v = self.project_qkv(x)
+        v = v.view(b, s, n, d)
         if self.qk_norm and self.fuse_qk_norm and x.dtype in (torch.bfloat16, torch.float32) \
                 and self.num_heads <= 64:
             # the two RMSNorms run inside the append kernel
-            q, k = self.q(x).view(b, s, n, d), self.k(x).view(b, s, n, d)
+            q, k = q.view(b, s, n, d), k.view(b, s, n, d)
             norm = (self.norm_q.weight.detach(), self.norm_k.weight.detach(), self.eps)
             out = self.attend(q, k, v, grid_sizes, freqs, kv_cache, current_start, qk_norm=norm)
         else:
-            q = self.norm_q(self.q(x)).view(b, s, n, d)
-            k = self.norm_k(self.k(x)).view(b, s, n, d)
+            q = self.norm_q(q).view(b, s, n, d)
+            k = self.norm_k(k).view(b, s, n, d)
             out = self.attend(q, k, v, grid_sizes, freqs, kv_cache, current_start)
         return self.o(out.flatten(2))
 
