@@ -545,6 +545,32 @@ def module_path_section(args, w, headline_ms):
     for m in mods:
         m.fuse_qkv_projection = False          # the reference's three launches, for comparison
     per_layer_apart = timed()
+    del mods, caches
+    # the text cross-attention of the same block (wan_base/modules/model.py:160-196): q projection and its
+    # norm, attention against the prompt's cached 512 keys, o projection
+    from streamdiffusionv2_amd.attention import WanT2VCrossAttention
+    cross = [WanT2VCrossAttention(dim, H).to(dev).to(w.dtype) for _ in range(layers)]
+    context = torch.randn(B, 512, dim, device=dev, generator=gen).to(w.dtype)
+    text_caches = [{"is_init": False, "k": None, "v": None} for _ in range(layers)]
+
+    def cross_step():
+        for layer in range(layers):
+            cross[layer](x, context, None, text_caches[layer])
+
+    with torch.no_grad():
+        for _ in range(args.warmup + 2):
+            cross_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            cross_step()
+        torch.cuda.synchronize()
+    cross_per_layer = (time.perf_counter() - t0) * 1e3 / (args.steps * layers)
+    out["cross_attention_forward"] = {
+        "ms_per_layer_call": cross_per_layer, "ms_per_step": cross_per_layer * w.layers, "layers_timed": layers,
+        "context_tokens": 512,
+        "what": "WanT2VCrossAttention.forward on the cached prompt: q projection (vendor GEMM), q RMSNorm (one launch "
+                "of the library), attention, o projection; scaled to the layer count"}
     out["module_forward"] = {"ms_per_layer_call": per_layer, "ms_per_step": per_layer * w.layers, "layers_timed": layers,
                              "ms_per_step_with_three_projection_launches": per_layer_apart * w.layers,
                              "what": "CausalWanSelfAttention.forward with its defaults: q / k / v as one vendor GEMM "

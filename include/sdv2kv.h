@@ -31,7 +31,7 @@
 extern "C" {
 #endif
 
-#define SDV2KV_ABI_VERSION 11
+#define SDV2KV_ABI_VERSION 12
 #define SDV2_HEAD_DIM 128      /* causal_stream_inference.py:99-100 fixes 128 */
 #define SDV2_MAX_ROWS 16       /* rows (B) per sdv2_kv_append_rope call       */
 #define SDV2_MAX_SINK_FRAMES 16 /* sink frames per sdv2_sink_similarity call  */
@@ -363,6 +363,36 @@ typedef struct sdv2_relayout_params {
 } sdv2_relayout_params;
 
 int sdv2_cache_relayout(const sdv2_relayout_params* p);
+
+/* ------------------------------------------------------------------------
+ * RMS norm over the model width, as a call of its own.
+ *
+ * Replaces WanRMSNorm.forward (models/wan/wan_base/modules/model.py:77-86)
+ * where the norm is not folded into sdv2_kv_append_rope: norm_q of the text
+ * cross-attention (model.py:181), and norm_q / norm_k of the self-attention
+ * when a caller applies them apart (causal_model.py:212-218):
+ *   out[t, :] = type_as(float(x[t, :]) * rsqrt(mean(float(x[t, :])^2) + eps)) * weight
+ * for every token t, with the three roundings of the torch expression.  The
+ * fp32 sum of squares is taken in the order of PyTorch's CPU sum kernel, as in
+ * sdv2_kv_append_rope, so the result is bit for bit the torch module's on the
+ * CPU.  width must be a multiple of 128, at most 64 * 128; rows are `width`
+ * contiguous elements, x_token_stride / out_token_stride elements apart (a
+ * slice of a wider projection output works); out may be x.
+ * ---------------------------------------------------------------------- */
+typedef struct sdv2_rms_norm_params {
+  const void* x;               /* [tokens, width]                              */
+  void* out;                   /* [tokens, width]                              */
+  const void* weight;          /* [width], the tensors' dtype                  */
+  int64_t x_token_stride;      /* elements                                     */
+  int64_t out_token_stride;
+  int64_t tokens;
+  int32_t width;
+  int32_t dtype;               /* sdv2_dtype of x, out and weight              */
+  float eps;
+  void* stream;                /* hipStream_t                                  */
+} sdv2_rms_norm_params;
+
+int sdv2_rms_norm(const sdv2_rms_norm_params* p);
 
 #ifdef __cplusplus
 }

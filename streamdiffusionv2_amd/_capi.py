@@ -12,7 +12,7 @@ from typing import Optional
 
 LIB_PATH = Path(__file__).resolve().parent / "_lib" / "libsdv2kv.so"
 
-ABI_VERSION = 11
+ABI_VERSION = 12
 HEAD_DIM = 128
 MAX_ROWS = 16
 
@@ -44,6 +44,7 @@ EXPORTED_SYMBOLS = (
     "sdv2_sink_frame_sums_bytes",
     "sdv2_sink_similarity",
     "sdv2_cache_relayout",
+    "sdv2_rms_norm",
     "sdv2_event_create",
     "sdv2_event_destroy",
     "sdv2_event_elapsed_ms",
@@ -137,6 +138,18 @@ class SinkSimParams(C.Structure):
     ]
 
 
+class RmsNormParams(C.Structure):
+    _fields_ = [
+        ("x", C.c_void_p), ("out", C.c_void_p), ("weight", C.c_void_p),
+        ("x_token_stride", C.c_int64), ("out_token_stride", C.c_int64),
+        ("tokens", C.c_int64),
+        ("width", C.c_int32),
+        ("dtype", C.c_int32),
+        ("eps", C.c_float),
+        ("stream", C.c_void_p),
+    ]
+
+
 class RelayoutParams(C.Structure):
     _fields_ = [
         ("src", C.c_void_p), ("dst", C.c_void_p),
@@ -194,6 +207,8 @@ def lib() -> C.CDLL:
     handle.sdv2_sink_similarity.argtypes = [C.POINTER(SinkSimParams)]
     handle.sdv2_cache_relayout.restype = C.c_int
     handle.sdv2_cache_relayout.argtypes = [C.POINTER(RelayoutParams)]
+    handle.sdv2_rms_norm.restype = C.c_int
+    handle.sdv2_rms_norm.argtypes = [C.POINTER(RmsNormParams)]
     handle.sdv2_event_create.restype = C.c_int
     handle.sdv2_event_create.argtypes = [C.POINTER(C.c_void_p)]
     handle.sdv2_event_destroy.restype = C.c_int

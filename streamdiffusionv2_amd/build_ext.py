@@ -17,7 +17,7 @@ CSRC = PKG_DIR / "csrc"
 LIB_DIR = PKG_DIR / "_lib"
 LIB_PATH = LIB_DIR / "libsdv2kv.so"
 SOURCES = ["sdv2kv_api.hip", "kv_append_rope.hip", "swa_attn_fwd.hip", "swa_attn_fwd_f32.hip", "sink_similarity.hip",
-           "cache_relayout.hip", "mfma_ceiling.hip"]
+           "cache_relayout.hip", "rms_norm.hip", "mfma_ceiling.hip"]
 
 # -packed-fp32-ops is switched off: the compiler would otherwise form
 # v_pk_*_f32 from ordinary float code.

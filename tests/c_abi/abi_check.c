@@ -67,6 +67,22 @@ int main(void) {
   rl.dst_global_end_index = (int64_t*)&rl;          /* destination index without a source */
   expect("relayout index without source", sdv2_cache_relayout(&rl), SDV2_ERR_INVALID_ARG);
 
+  sdv2_rms_norm_params rn;
+  expect("rms_norm(NULL)", sdv2_rms_norm(NULL), SDV2_ERR_INVALID_ARG);
+  memset(&rn, 0, sizeof rn);
+  rn.width = 100;
+  expect("rms_norm width 100", sdv2_rms_norm(&rn), SDV2_ERR_UNSUPPORTED);
+  rn.width = 65 * SDV2_HEAD_DIM;
+  expect("rms_norm width 65 * 128", sdv2_rms_norm(&rn), SDV2_ERR_UNSUPPORTED);
+  rn.width = 12 * SDV2_HEAD_DIM;
+  expect("rms_norm of nothing", sdv2_rms_norm(&rn), SDV2_OK);
+  rn.tokens = 4;
+  expect("rms_norm null tensors", sdv2_rms_norm(&rn), SDV2_ERR_INVALID_ARG);
+  rn.x = &rn; rn.out = &rn; rn.weight = &rn;                    /* (never launched: the stride below is refused) */
+  rn.x_token_stride = 8;
+  rn.out_token_stride = rn.width;
+  expect("rms_norm rows that overlap", sdv2_rms_norm(&rn), SDV2_ERR_INVALID_ARG);
+
   /* struct layouts, for the bindings to compare themselves with */
   printf("layout sdv2_append_params size=%zu stream=%zu q_inv_rms=%zu\n", sizeof(sdv2_append_params),
          offsetof(sdv2_append_params, stream), offsetof(sdv2_append_params, q_inv_rms));
@@ -74,6 +90,8 @@ int main(void) {
          offsetof(sdv2_attn_params, stream), offsetof(sdv2_attn_params, q_inv_rms));
   printf("layout sdv2_sink_sim_params size=%zu stream=%zu planned_frame=%zu\n", sizeof(sdv2_sink_sim_params),
          offsetof(sdv2_sink_sim_params, stream), offsetof(sdv2_sink_sim_params, planned_frame));
+  printf("layout sdv2_rms_norm_params size=%zu stream=%zu eps=%zu\n", sizeof(sdv2_rms_norm_params),
+         offsetof(sdv2_rms_norm_params, stream), offsetof(sdv2_rms_norm_params, eps));
   printf("layout sdv2_relayout_params size=%zu stream=%zu global_end_shift=%zu\n", sizeof(sdv2_relayout_params),
          offsetof(sdv2_relayout_params, stream), offsetof(sdv2_relayout_params, global_end_shift));
 

@@ -203,6 +203,7 @@ def test_plain_c_caller(tmp_path):
     for c_name, binding, last in (("sdv2_append_params", _capi.AppendParams, "q_inv_rms"),
                                   ("sdv2_attn_params", _capi.AttnParams, "q_inv_rms"),
                                   ("sdv2_sink_sim_params", _capi.SinkSimParams, "planned_frame"),
+                                  ("sdv2_rms_norm_params", _capi.RmsNormParams, "eps"),
                                   ("sdv2_relayout_params", _capi.RelayoutParams, "global_end_shift")):
         m = re.search(rf"layout {c_name} size=(\d+) stream=(\d+) {last}=(\d+)", run.stdout)
         assert m, run.stdout
