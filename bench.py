@@ -241,17 +241,27 @@ def gpu_bench(args, w):
         step()
     torch.cuda.synchronize()
 
-    marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        marks[i].record()
-        step()
-    marks[args.steps].record()
-    torch.cuda.synchronize()
-    t1 = time.perf_counter()
-    ms_per_step = (t1 - t0) * 1e3 / args.steps
-    per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
-    ms_median = per_step[len(per_step) // 2]
+    # The timed pass: exactly args.steps steps between two synchronisations.  A pass that an outside stall
+    # hit (another process sampling the GPU, an allocator refill: its mean then lies far above the median of
+    # its own steps) says nothing about the path; it is reported as discarded and the pass is taken again,
+    # at most twice.
+    discarded = []
+    for attempt in range(3):
+        marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            marks[i].record()
+            step()
+        marks[args.steps].record()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        ms_per_step = (t1 - t0) * 1e3 / args.steps
+        per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
+        ms_median = per_step[len(per_step) // 2]
+        if ms_per_step <= 1.25 * ms_median or args.steps < 4:
+            break
+        discarded.append({"ms_per_step": ms_per_step, "ms_per_step_median": ms_median, "slowest_step_ms": per_step[-1]})
 
     # instrumented pass over the same steps: per-kernel durations
     timers = []
@@ -286,6 +296,7 @@ def gpu_bench(args, w):
     return {
         "ms_per_step": ms_per_step,
         "ms_median": ms_median,
+        "discarded": discarded,
         "fill_ms": fill_ms,
         "append_ms": t_append,
         "attn_ms": t_attn,
@@ -604,7 +615,21 @@ def qk_norm_section(args, w):
         c = caches[i % layers]
         ops.kv_append_rope(q, k, v, c["k"], c["v"], table, w.grid, starts, dst, q_out=q_out, qk_norm=weights)
 
+    def torch_norm(x, weight):
+        # WanRMSNorm.forward as the reference writes it (wan_base/modules/model.py:77-86), in stock torch
+        xf = x.float()
+        return (xf * torch.rsqrt(xf.pow(2).mean(dim=-1, keepdim=True) + 1e-6)).type_as(x) * weight
+
     def unfused(i):
+        q, k, v = qkv[i % layers]
+        c = caches[i % layers]
+        with torch.no_grad():
+            qn = torch_norm(q.flatten(2), weights[0]).view_as(q)
+            kn = torch_norm(k.flatten(2), weights[1]).view_as(k)
+        ops.kv_append_rope(qn, kn, v, c["k"], c["v"], table, w.grid, starts, dst, q_out=q_out)
+
+    def library_norms(i):
+        # the norms as modules of their own, each one launch of the library's kernel
         q, k, v = qkv[i % layers]
         c = caches[i % layers]
         with torch.no_grad():
@@ -614,7 +639,8 @@ def qk_norm_section(args, w):
 
     out = {}
     n = 4 * layers
-    for name, fn in (("fused_ms", fused), ("torch_norms_plus_append_ms", unfused)):
+    for name, fn in (("fused_ms", fused), ("torch_norms_plus_append_ms", unfused),
+                     ("library_norm_launches_plus_append_ms", library_norms)):
         for i in range(layers):
             fn(i)
         torch.cuda.synchronize()
@@ -647,9 +673,20 @@ def qk_norm_section(args, w):
         out[name + "_ms"] = sum(kernel_ms) / len(kernel_ms)
         out[name + "_bytes"] = moved
         out[name + "_GBps"] = moved / (out[name + "_ms"] * 1e-3) / 1e9
+    # the norm as a launch of its own (sdv2_rms_norm): read and write B * S * H * 128 elements
+    flat = qkv[0][0].flatten(2)
+    norm_bytes = 2 * flat.numel() * flat.element_size()
+    kernel_ms = []
+    for i in range(n):
+        timer.arm(_capi.KERNEL_NORM)
+        ops.rms_norm(qkv[i % layers][0].flatten(2), weights[0], 1e-6)
+        kernel_ms.append(timer.elapsed_ms())
+    out["rms_norm_kernel_ms"] = sum(kernel_ms) / len(kernel_ms)
+    out["rms_norm_kernel_bytes"] = norm_bytes
+    out["rms_norm_kernel_GBps"] = norm_bytes / (out["rms_norm_kernel_ms"] * 1e-3) / 1e9
     timer.close()
-    out["note"] = ("fused_ms / torch_norms_plus_append_ms are host-inclusive per-call times (the torch path launches "
-                   "about a dozen kernels per call); fused_kernel_ms is the kernel alone")
+    out["note"] = ("fused_ms / torch_norms_plus_append_ms / library_norm_launches_plus_append_ms are host-inclusive "
+                   "per-call times (the torch path launches about a dozen kernels per call); *_kernel_ms are kernels alone")
     # The consumer side (causal_model.py:387-389): the o projection reads the attention output in place.
     # Per layer: attention alone, the vendor GEMM alone, and the two back to back on one stream.
     dim = H * 128
@@ -1024,6 +1061,9 @@ def main():
         "warmup": args.warmup,
         "ms_per_step": g["ms_per_step"],
         "ms_per_step_median": g["ms_median"],
+        # timed passes thrown away because an outside stall hit them (mean above 1.25 x the pass's own median
+        # step); empty in a normal run
+        "timed_passes_discarded": g["discarded"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,

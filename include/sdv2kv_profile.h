@@ -22,7 +22,8 @@ typedef enum sdv2_profile_kernel {
   SDV2_KERNEL_RELAYOUT = 2,    /* sdv2_cache_relayout                          */
   SDV2_KERNEL_SINK = 3,        /* sdv2_sink_similarity                         */
   SDV2_KERNEL_COPY = 4,        /* sdv2_copy_bytes                              */
-  SDV2_KERNEL_COUNT = 5
+  SDV2_KERNEL_NORM = 5,        /* sdv2_rms_norm                                */
+  SDV2_KERNEL_COUNT = 6
 } sdv2_profile_kernel;
 
 /* ------------------------------------------------------------------------

@@ -28,7 +28,7 @@ STATIC_SCRATCH_BYTES = 64 << 20
 DTYPE_BF16 = 0
 DTYPE_F32 = 1
 
-KERNEL_APPEND, KERNEL_ATTENTION, KERNEL_RELAYOUT, KERNEL_SINK, KERNEL_COPY = range(5)
+KERNEL_APPEND, KERNEL_ATTENTION, KERNEL_RELAYOUT, KERNEL_SINK, KERNEL_COPY, KERNEL_NORM = range(6)
 STREAM_REGISTERS, STREAM_LDS_32_ROWS, STREAM_LDS_64_ROWS, STREAM_ATTENTION_MIX, STREAM_ATTENTION_MIX_64_ROWS = range(5)
 
 # every symbol include/sdv2kv.h and include/sdv2kv_profile.h declare

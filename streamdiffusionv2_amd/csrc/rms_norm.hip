@@ -17,6 +17,7 @@
 #include <type_traits>
 
 #include "sdv2kv.h"
+#include "sdv2kv_profile.h"
 #include "sdv2kv_internal.h"
 #include "rope_device.h"
 
@@ -102,8 +103,8 @@ extern "C" int sdv2_rms_norm(const sdv2_rms_norm_params* p) {
   const int steps = (a.heads + 3) / 4;
   auto launch = [&](auto steps_c) {
     constexpr int kS = decltype(steps_c)::value;
-    if (p->dtype == SDV2_BF16) hipLaunchKernelGGL((rms_norm_kernel<uint16_t, kS>), grid, block, 0, stream, a);
-    else hipLaunchKernelGGL((rms_norm_kernel<float, kS>), grid, block, 0, stream, a);
+    if (p->dtype == SDV2_BF16) sdv2::launch_timed(SDV2_KERNEL_NORM, rms_norm_kernel<uint16_t, kS>, grid, block, 0, stream, a);
+    else sdv2::launch_timed(SDV2_KERNEL_NORM, rms_norm_kernel<float, kS>, grid, block, 0, stream, a);
   };
   if (steps <= 3) launch(std::integral_constant<int, 3>{});
   else if (steps <= 10) launch(std::integral_constant<int, 10>{});
