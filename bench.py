@@ -12,6 +12,7 @@ stream) and the CPU oracle timed on the host cores of the same box.
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import os
 import sys
@@ -248,6 +249,7 @@ def gpu_bench(args, w):
     discarded = []
     for attempt in range(3):
         marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
+        gc.collect()                 # (a collection of the interpreter's in the middle of a 60 ms pass would be such a stall)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for i in range(args.steps):
