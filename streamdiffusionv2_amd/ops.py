@@ -49,6 +49,24 @@ def _current_device_index() -> int:
     return torch.cuda.current_device()
 
 
+class _NoSwitch:
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on_device(dev: torch.device):
+    """Context in which ``dev`` is the current device: torch's guard when it is
+    another one, nothing at all (the usual case, and several microseconds less
+    per call) when it already is."""
+    return _NO_SWITCH if torch.cuda.current_device() == dev.index else torch.cuda.device(dev)
+
+
 def _i64_array(values: Sequence[int]):
     return (C.c_int64 * len(values))(*[int(v) for v in values])
 
@@ -164,7 +182,7 @@ def kv_append_rope(
 
     lib = _capi.lib()
     stream = _stream_ptr(dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         for r0 in range(0, rows, _capi.MAX_ROWS):
             r1 = min(rows, r0 + _capi.MAX_ROWS)
             p = _capi.AppendParams()
@@ -247,7 +265,7 @@ def causal_rope_apply(x: torch.Tensor, grid_sizes, freqs: torch.Tensor, start_fr
         raise RuntimeError("x must be dense (its copy did not keep the strides)")
 
     lib = _capi.lib()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         r0 = 0
         while r0 < len(grids):
             r1 = r0 + 1
@@ -435,7 +453,7 @@ def swa_attention(
                 or inv_rms.device != dev:
             raise RuntimeError(f"q_inv_rms must be a contiguous float32 tensor of {rows} x {q_tokens} elements on {dev}")
         p.q_norm_weight, p.q_inv_rms = weight.data_ptr(), inv_rms.data_ptr()
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         if static_scratch:
             _capi.check(lib.sdv2_swa_attn_fwd_static(C.byref(p)), "sdv2_swa_attn_fwd_static")
         else:
@@ -553,7 +571,7 @@ def sink_similarity(
         p.frame_sums = frame_sums.data_ptr()
         p.stale_frames = C.cast(stale, C.POINTER(C.c_uint32))
         p.planned_frame = C.cast(planned, C.POINTER(C.c_int32))
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _capi.check(lib.sdv2_sink_similarity(C.byref(p)), "sdv2_sink_similarity")
     return similarity, refresh
 
@@ -869,7 +887,7 @@ def cache_relayout(
     p.stream = _stream_ptr(dev)
     if timer is not None:
         timer.arm(_capi.KERNEL_RELAYOUT)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _capi.check(_capi.lib().sdv2_cache_relayout(C.byref(p)), "sdv2_cache_relayout")
 
 
@@ -922,7 +940,7 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[to
     p.x_token_stride, p.out_token_stride = x_step, out_step
     p.tokens, p.width, p.dtype, p.eps = tokens, width, _DTYPES[x.dtype], float(eps)
     p.stream = _stream_ptr(dev)
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _capi.check(_capi.lib().sdv2_rms_norm(C.byref(p)), "sdv2_rms_norm")
     return out
 
@@ -934,5 +952,5 @@ def copy_bytes(dst: torch.Tensor, src: torch.Tensor) -> None:
     n = src.numel() * src.element_size()
     if dst.numel() * dst.element_size() != n or not dst.is_contiguous() or not src.is_contiguous():
         raise RuntimeError("copy_bytes needs contiguous tensors of equal byte size")
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _capi.check(_capi.lib().sdv2_copy_bytes(dst.data_ptr(), src.data_ptr(), n, _stream_ptr(dev)), "sdv2_copy_bytes")
