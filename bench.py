@@ -238,9 +238,6 @@ def gpu_bench(args, w):
             if not args.zero_inputs:
                 phys.copy_(torch.randn(phys.shape, generator=gen, device=dev, dtype=torch.float32) * w.input_scale)
     state["call"] = fill_calls
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
 
     # The timed pass: exactly args.steps steps between two synchronisations.  A pass that an outside stall
     # hit (another process sampling the GPU, an allocator refill: its mean then lies far above the median of
@@ -249,15 +246,24 @@ def gpu_bench(args, w):
     discarded = []
     for attempt in range(3):
         marks = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps + 1)]
-        gc.collect()                 # (a collection of the interpreter's in the middle of a 60 ms pass would be such a stall)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for i in range(args.steps):
-            marks[i].record()
-            step()
-        marks[args.steps].record()
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
+        # The interpreter's garbage collection stays out of the pass (a collection in the middle of 60 ms
+        # would be such a stall) and is run before the warm-up, not after it: the GPU must not sit idle
+        # for tens of milliseconds right before the clock starts, or the first steps run at idle clocks.
+        gc.collect()
+        gc.disable()
+        try:
+            for _ in range(args.warmup):
+                step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(args.steps):
+                marks[i].record()
+                step()
+            marks[args.steps].record()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+        finally:
+            gc.enable()
         ms_per_step = (t1 - t0) * 1e3 / args.steps
         per_step = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(args.steps))
         ms_median = per_step[len(per_step) // 2]
@@ -298,6 +304,7 @@ def gpu_bench(args, w):
     return {
         "ms_per_step": ms_per_step,
         "ms_median": ms_median,
+        "ms_slowest": per_step[-1],
         "discarded": discarded,
         "fill_ms": fill_ms,
         "append_ms": t_append,
@@ -1063,6 +1070,7 @@ def main():
         "warmup": args.warmup,
         "ms_per_step": g["ms_per_step"],
         "ms_per_step_median": g["ms_median"],
+        "ms_slowest_step": g["ms_slowest"],
         # timed passes thrown away because an outside stall hit them (mean above 1.25 x the pass's own median
         # step); empty in a normal run
         "timed_passes_discarded": g["discarded"],
