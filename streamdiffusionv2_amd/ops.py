@@ -891,12 +891,38 @@ def cache_relayout(
         _capi.check(_capi.lib().sdv2_cache_relayout(C.byref(p)), "sdv2_cache_relayout")
 
 
+def _norm_rows(t: torch.Tensor):
+    """(rows, elements between rows) of a tensor [..., width] whose rows are
+    contiguous and evenly spaced, else None."""
+    width = t.shape[-1]
+    if width > 1 and t.stride(-1) != 1:
+        return None
+    rows = t.numel() // width
+    if t.dim() == 1 or rows <= 1:
+        return rows, width
+    step = expect = None
+    for size, stride in zip(reversed(t.shape[:-1]), reversed(t.stride()[:-1])):
+        if size == 1:
+            continue
+        if step is None:
+            step = expect = stride
+        elif stride != expect:
+            return None
+        expect *= size
+    if step is None or step < width or step % 8 != 0:
+        return None
+    return rows, step
+
+
 def rms_norm_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
     """Can :func:`rms_norm` take this input?  (A device tensor of a dtype the
-    library knows, rows of a multiple of 128 up to 8192 contiguous elements.)"""
+    library knows; rows of a multiple of 128 up to 8192 contiguous elements, 16-byte
+    aligned and evenly spaced; a contiguous weight of the same dtype.)"""
     width = x.shape[-1] if x.dim() else 0
     return (x.is_cuda and x.dtype in _DTYPES and weight.dtype == x.dtype and weight.device == x.device
-            and width > 0 and width % HEAD_DIM == 0 and width // HEAD_DIM <= 64 and weight.numel() == width)
+            and width > 0 and width % HEAD_DIM == 0 and width // HEAD_DIM <= 64 and weight.numel() == width
+            and weight.is_contiguous() and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0
+            and _norm_rows(x) is not None)
 
 
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -908,36 +934,21 @@ def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float, out: Optional[to
     tensor and may be x itself."""
     dev = _require_gpu(x, weight)
     if not rms_norm_supported(x, weight):
-        raise RuntimeError(f"rms_norm takes bf16 / fp32 rows of a multiple of 128 up to 8192 elements with a weight of "
-                           f"the same dtype and width, got x {tuple(x.shape)} {x.dtype}, weight {tuple(weight.shape)} {weight.dtype}")
+        raise RuntimeError(f"rms_norm takes bf16 / fp32 rows of a multiple of 128 up to 8192 contiguous, 16-byte aligned, "
+                           f"evenly spaced elements with a contiguous weight of the same dtype and width, got x "
+                           f"{tuple(x.shape)} {x.dtype} strides {x.stride()}, weight {tuple(weight.shape)} {weight.dtype}")
     width = x.shape[-1]
-
-    def rows_of(t: torch.Tensor, name: str):
-        """(tokens, elements between rows) of a tensor whose leading dimensions walk rows evenly."""
-        if t.stride(-1) != 1 and width > 1:
-            raise RuntimeError(f"{name}: the last dimension must be contiguous")
-        tokens = t.numel() // width
-        if t.dim() == 1 or tokens <= 1:
-            return tokens, width
-        step = t.stride(-2)
-        expect = step
-        for size, stride in zip(reversed(t.shape[:-1]), reversed(t.stride()[:-1])):
-            if size != 1 and stride != expect:
-                raise RuntimeError(f"{name}: rows must be evenly spaced (shape {tuple(t.shape)}, strides {t.stride()})")
-            expect *= size
-        return tokens, step
-
-    if not weight.is_contiguous():
-        raise RuntimeError("the norm weight must be contiguous")
-    tokens, x_step = rows_of(x, "x")
+    tokens, x_step = _norm_rows(x)
     if out is None:
         out = torch.empty(x.shape, dtype=x.dtype, device=dev)
     elif out.shape != x.shape or out.dtype != x.dtype or out.device != dev:
         raise RuntimeError("out must have x's shape, dtype and device")
-    _, out_step = rows_of(out, "out")
+    rows = _norm_rows(out)
+    if rows is None or out.data_ptr() % 16:
+        raise RuntimeError("out: rows must be contiguous, 16-byte aligned and evenly spaced")
     p = _capi.RmsNormParams()
     p.x, p.out, p.weight = x.data_ptr(), out.data_ptr(), weight.data_ptr()
-    p.x_token_stride, p.out_token_stride = x_step, out_step
+    p.x_token_stride, p.out_token_stride = x_step, rows[1]
     p.tokens, p.width, p.dtype, p.eps = tokens, width, _DTYPES[x.dtype], float(eps)
     p.stream = _stream_ptr(dev)
     with _on_device(dev):
