@@ -52,6 +52,23 @@ def test_rows_inside_a_wider_tensor_and_in_place(gpu_device):
 
 
 @pytest.mark.gpu
+def test_fp32_rows_inside_a_wider_tensor(gpu_device):
+    print("rms norm on an fp32 slice", flush=True)
+    gen = torch.Generator().manual_seed(13)
+    width, tokens = 640, 37
+    wide = torch.randn(3, tokens, 2 * width, generator=gen) * 4.0
+    weight = torch.rand(width, generator=gen) + 0.5
+    want = oracle.wan_rms_norm(wide[..., width:], weight, 1e-5)
+    dev = wide.to(gpu_device)
+    got = ops.rms_norm(dev[..., width:], weight.to(gpu_device), 1e-5)
+    assert torch.equal(_bits(got.cpu()), _bits(want))
+    ops.rms_norm(dev[..., width:], weight.to(gpu_device), 1e-5, out=dev[..., :width])      # into the other half
+    after = dev.cpu()
+    assert torch.equal(_bits(after[..., :width]), _bits(want))
+    assert torch.equal(_bits(after[..., width:]), _bits(wide[..., width:]))
+
+
+@pytest.mark.gpu
 def test_the_module_uses_the_kernel_and_keeps_the_expression_elsewhere(gpu_device):
     print("WanRMSNorm module", flush=True)
     torch.manual_seed(12)

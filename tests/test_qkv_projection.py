@@ -102,6 +102,15 @@ def test_watched_or_wrapped_layers_are_called_themselves():
         assert torch.equal(v, wrapped(x))
 
 
+def test_linears_without_bias_pack_without_one():
+    torch.manual_seed(6)
+    mod = CausalWanSelfAttention(256, 2)
+    for layer in (mod.q, mod.k, mod.v):
+        layer.bias = None
+    x = torch.randn(2, 3, 256)
+    assert _close(mod, x) and mod._packed is not None and mod._packed[2] is None
+
+
 def test_a_module_made_under_inference_mode_packs_too():
     with torch.inference_mode():
         mod = CausalWanSelfAttention(256, 2)
